@@ -9,6 +9,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "../kernels/mix_linrec.h"
+
 namespace rfqmix {
 void launch_embed_sinusoid(bool, const int32_t*, const int32_t*, const void*, const float*, float,
                            float*, int, int, int, hipStream_t);
@@ -63,6 +65,22 @@ void launch_moe_pair_up(bool, const void*, int64_t, const int32_t*, const void*,
                         int, int, int, hipStream_t);
 void launch_moe_pair_down(bool, const void*, const int32_t*, const float*, const void*, const void*,
                           int64_t, float*, int, int, int, int, int, hipStream_t);
+void launch_residual_add_norm(bool, float*, const void*, int64_t, bool, const void*, int64_t, bool,
+                              const float*, const float*, float, float, void*, int, int,
+                              hipStream_t);
+void launch_rotary_append(bool, const void*, int64_t, const int32_t*, const float*, int,
+                          const int32_t*, void*, void*, int, int, int, int, int, int, int, int64_t,
+                          float*, hipStream_t);
+void launch_conv_act_heads(bool, const void*, int64_t, const float*, float*, const int32_t*,
+                           const int32_t*, const int32_t*, const int32_t*, float*, int, int, int,
+                           int, int, int, float, hipStream_t);
+void launch_moe_route_topk(const float*, const float*, int, int, int, int32_t*, float*, hipStream_t);
+void launch_gelu_rows(bool, const void*, int64_t, void*, int64_t, int, int, hipStream_t);
+size_t attn_diff_lds(int);
+bool launch_attn_diff_window(bool, const float*, const void*, const void*, const int32_t*, int,
+                             const int32_t*, const int32_t*, const int32_t*, const int32_t*,
+                             const int32_t*, int, const void*, int64_t, void*, int64_t, float, int,
+                             float, float, float, int, int, int, int, int, hipStream_t);
 }  // namespace rfqmix
 
 namespace {
@@ -475,6 +493,195 @@ void moe_pair_down(const Tensor& act, const Tensor& ids, const Tensor& weights, 
                                const_cast<float*>(f32p(out, "out")), T, top, d, F, E, stream());
 }
 
+// ---- parallel-sublayer layers: residual, rotary differential attention, linear recurrences
+void residual_add_norm(const Tensor& x, const OptT& y1, const OptT& y2, const OptT& shift,
+                       const OptT& w, double eps, double offset, const OptT& out) {
+  TORCH_CHECK(x.dim() == 2, "residual_add_norm: x [T, d]");
+  const int T = (int)x.size(0), d = (int)x.size(1);
+  const void* yp[2] = {nullptr, nullptr};
+  int64_t ys[2] = {0, 0};
+  bool yf[2] = {true, true};
+  const OptT* yy[2] = {&y1, &y2};
+  for (int i = 0; i < 2; ++i)
+    if (yy[i]->has_value()) {
+      const Tensor& y = **yy[i];
+      yf[i] = act_f32(y, "residual_add_norm y");
+      TORCH_CHECK(rows2d(y, T, d), "residual_add_norm: y [T, d]");
+      yp[i] = y.data_ptr();
+      ys[i] = y.stride(0);
+    }
+  bool of32 = true;
+  void* op = nullptr;
+  if (w.has_value()) {
+    TORCH_CHECK(out.has_value(), "residual_add_norm: a norm weight needs out");
+    of32 = act_f32(*out, "residual_add_norm out");
+    TORCH_CHECK(rows2d(*out, T, d) && out->is_contiguous(), "residual_add_norm: out [T, d]");
+    op = out->data_ptr();
+  }
+  rfqmix::launch_residual_add_norm(of32, const_cast<float*>(f32p(x, "x")), yp[0], ys[0], yf[0],
+                                   yp[1], ys[1], yf[1], optf(shift, "shift", d), optf(w, "w", d),
+                                   (float)eps, (float)offset, op, T, d, stream());
+}
+
+void rotary_append(const Tensor& qkv, const Tensor& pos, const Tensor& inv_freq,
+                   const Tensor& slots, const Tensor& k_cache, const Tensor& v_cache, int64_t H,
+                   int64_t G, int64_t maps, int64_t dim, int64_t vdim, const Tensor& q_out) {
+  const bool f32 = act_f32(qkv, "rotary_append qkv");
+  TORCH_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1, "rotary_append: qkv [T, N]");
+  const int T = (int)qkv.size(0);
+  const int64_t kw = maps * dim;
+  TORCH_CHECK(H >= 1 && G >= 1 && maps >= 1 && dim >= 1 && vdim >= 1 &&
+              qkv.size(1) >= (H + G) * kw + G * vdim, "rotary_append: qkv narrower than q | k | v");
+  TORCH_CHECK(k_cache.is_cuda() && v_cache.is_cuda() && k_cache.scalar_type() == qkv.scalar_type() &&
+              v_cache.scalar_type() == qkv.scalar_type() && k_cache.is_contiguous() &&
+              v_cache.is_contiguous() && k_cache.dim() == 4 && v_cache.dim() == 4 &&
+              k_cache.size(1) == G && k_cache.size(3) == kw && v_cache.size(1) == G &&
+              v_cache.size(3) == vdim && v_cache.size(0) == k_cache.size(0) &&
+              v_cache.size(2) == k_cache.size(2),
+              "rotary_append: k_cache [blocks, G, BS, maps dim], v_cache [blocks, G, BS, vdim]");
+  const int nrot = (int)inv_freq.numel();
+  TORCH_CHECK(2 * nrot <= dim, "rotary_append: more rotated dimensions than a map has");
+  TORCH_CHECK(q_out.dim() == 3 && q_out.size(0) == T && q_out.size(1) == H && q_out.size(2) == kw,
+              "rotary_append: q_out [T, H, maps dim]");
+  const float* fr = nrot > 0 ? f32p(inv_freq, "inv_freq") : nullptr;
+  rfqmix::launch_rotary_append(f32, qkv.data_ptr(), qkv.stride(0), i32p(pos, "positions", T), fr,
+                               nrot, i32p(slots, "slots", T), k_cache.data_ptr(),
+                               v_cache.data_ptr(), T, (int)H, (int)G, (int)maps, (int)dim,
+                               (int)vdim, (int)k_cache.size(2),
+                               k_cache.size(0) * k_cache.size(2),
+                               const_cast<float*>(f32p(q_out, "q_out")), stream());
+}
+
+void attn_diff_window(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache,
+                      const Tensor& bt, const Tensor& q_start, const Tensor& q_len,
+                      const Tensor& kv_len, const Tensor& work_seq, const Tensor& work_qblk,
+                      const Tensor& gate, const Tensor& out, double scale, int64_t window,
+                      double lam, double eps, double out_mult) {
+  const bool f32 = act_f32(k_cache, "attn_diff_window k_cache");
+  TORCH_CHECK(q.dim() == 3 && q.size(2) % 2 == 0, "attn_diff_window: q [T, H, 2 dim]");
+  const int T = (int)q.size(0), H = (int)q.size(1), dim = (int)q.size(2) / 2;
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.is_contiguous() &&
+              v_cache.is_contiguous() && v_cache.is_cuda() &&
+              v_cache.scalar_type() == k_cache.scalar_type() && k_cache.size(3) == 2 * dim &&
+              v_cache.size(1) == k_cache.size(1) && v_cache.size(0) == k_cache.size(0) &&
+              v_cache.size(2) == k_cache.size(2),
+              "attn_diff_window: k_cache [blocks, G, BS, 2 dim], v_cache [blocks, G, BS, vdim]");
+  const int G = (int)k_cache.size(1), BS = (int)k_cache.size(2), vdim = (int)v_cache.size(3);
+  TORCH_CHECK(G >= 1 && H % G == 0 && H <= 65535, "attn_diff_window: H a multiple of G");
+  const int NB = (int)q_len.numel(), W = (int)work_seq.numel();
+  TORCH_CHECK(bt.dim() == 2 && bt.size(0) == NB, "attn_diff_window: block_tables [NB, maxb]");
+  TORCH_CHECK(work_qblk.numel() >= W, "attn_diff_window: work lists");
+  TORCH_CHECK(gate.is_cuda() && gate.scalar_type() == k_cache.scalar_type() && rows2d(gate, T, H),
+              "attn_diff_window: gate [T, H] in the cache's type");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == k_cache.scalar_type() &&
+              rows2d(out, T, (int64_t)H * vdim), "attn_diff_window: out [T, H vdim]");
+  TORCH_CHECK(window >= 0, "attn_diff_window: window");
+  const bool ok = rfqmix::launch_attn_diff_window(
+      f32, f32p(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), i32p(bt, "block_tables", 0),
+      (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
+      i32p(kv_len, "kv_len", NB), i32p(work_seq, "work_seq", W), i32p(work_qblk, "work_qblk", W), W,
+      gate.data_ptr(), gate.stride(0), out.data_ptr(), out.stride(0), (float)scale, (int)window,
+      (float)lam, (float)eps, (float)out_mult, H, G, dim, vdim, BS, stream());
+  TORCH_CHECK(ok, "attn_diff_window: value size too large for the LDS");
+}
+
+void conv_act_heads(const Tensor& x, const Tensor& w, const Tensor& state, const Tensor& row_state,
+                    const Tensor& row_back, const Tensor& row_fwd, const Tensor& pos,
+                    int64_t n_unit, int64_t dim, double unit_eps, const Tensor& out) {
+  const bool f32 = act_f32(x, "conv_act_heads x");
+  TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1 && w.dim() == 2 && state.dim() == 3,
+              "conv_act_heads: x [T, C], w [C, taps], state [2S, taps-1, C]");
+  const int T = (int)x.size(0), C = (int)x.size(1), taps = (int)w.size(1);
+  TORCH_CHECK(w.size(0) == C && taps >= 1, "conv_act_heads: w [C, taps]");
+  TORCH_CHECK(state.size(0) % 2 == 0 && state.size(1) == taps - 1 && state.size(2) == C,
+              "conv_act_heads: state [2S, taps-1, C]");
+  TORCH_CHECK(n_unit >= 0 && dim >= 1 && n_unit * dim <= C, "conv_act_heads: unit heads");
+  TORCH_CHECK((int64_t)C * 4 <= 64 * 1024, "conv_act_heads: too many channels for the LDS");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == C, "conv_act_heads: out [T, C]");
+  rfqmix::launch_conv_act_heads(f32, x.data_ptr(), x.stride(0), f32p(w, "w"),
+                                const_cast<float*>(f32p(state, "state")),
+                                i32p(row_state, "row_state", T), i32p(row_back, "row_back", T),
+                                i32p(row_fwd, "row_fwd", T), i32p(pos, "positions", T),
+                                const_cast<float*>(f32p(out, "out")), T, C, taps,
+                                (int)state.size(0) / 2, (int)n_unit, (int)dim, (float)unit_eps,
+                                stream());
+}
+
+void gated_linear_recurrence(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& z,
+                             const Tensor& rate, const Tensor& zbias, double zsign,
+                             const OptT& beta, const Tensor& gate, bool gate_sigmoid,
+                             const Tensor& norm_w, double eps, double q_scale, const Tensor& state,
+                             const Tensor& row_state, const Tensor& row_back, const Tensor& row_fwd,
+                             const Tensor& pos, const OptT& run_rows, const Tensor& out) {
+  const bool in_f32 = act_f32(q, "gated_linear_recurrence q");
+  const bool a_f32 = act_f32(out, "gated_linear_recurrence out");
+  TORCH_CHECK(state.dim() == 4 && state.size(0) % 2 == 0,
+              "gated_linear_recurrence: state [2 slots, H, dim, vdim]");
+  const int H = (int)state.size(1), dim = (int)state.size(2), vdim = (int)state.size(3);
+  TORCH_CHECK(q.dim() == 3 && k.dim() == 3 && v.dim() == 3 && q.stride(2) == 1 &&
+              k.stride(2) == 1 && v.stride(2) == 1 && k.scalar_type() == q.scalar_type() &&
+              v.scalar_type() == q.scalar_type() && k.is_cuda() && v.is_cuda(),
+              "gated_linear_recurrence: q, k [T, Hq, dim], v [T, H, vdim] of one type");
+  const int T = (int)q.size(0), Hq = (int)q.size(1);
+  TORCH_CHECK(Hq >= 1 && H % Hq == 0 && q.size(2) == dim && k.size(0) == T && k.size(1) == Hq &&
+              k.size(2) == dim && v.size(0) == T && v.size(1) == H && v.size(2) == vdim &&
+              q.stride(1) == dim && k.stride(1) == dim && v.stride(1) == vdim,
+              "gated_linear_recurrence: head counts and sizes of q, k, v");
+  TORCH_CHECK(z.is_cuda() && z.scalar_type() == at::kFloat && rows2d(z, T, (int64_t)H * dim),
+              "gated_linear_recurrence: z [T, H dim] float32");
+  TORCH_CHECK(gate.is_cuda() && gate.scalar_type() == out.scalar_type() &&
+              rows2d(gate, T, (int64_t)H * vdim), "gated_linear_recurrence: gate [T, H vdim]");
+  TORCH_CHECK(rows2d(out, T, (int64_t)H * vdim) && out.is_contiguous(),
+              "gated_linear_recurrence: out [T, H vdim]");
+  TORCH_CHECK(rfqmix::linrec_ok(dim, vdim) && H <= 65535,
+              "gated_linear_recurrence: head sizes outside the kernel's range");
+  rfqmix::LinrecArgs a;
+  a.q = q.data_ptr(); a.k = k.data_ptr(); a.v = v.data_ptr();
+  a.qs = q.stride(0); a.ks = k.stride(0); a.vs = v.stride(0);
+  a.z = z.data_ptr<float>(); a.zs = z.stride(0);
+  a.rate = f32p(rate, "rate", H); a.zbias = f32p(zbias, "zbias", (int64_t)H * dim);
+  a.zsign = (float)zsign;
+  a.beta = nullptr; a.bs = 0;
+  if (beta.has_value()) {
+    TORCH_CHECK(beta->is_cuda() && beta->scalar_type() == out.scalar_type() && rows2d(*beta, T, H),
+                "gated_linear_recurrence: beta [T, H]");
+    a.beta = beta->data_ptr(); a.bs = beta->stride(0);
+  }
+  a.gate = gate.data_ptr(); a.gs = gate.stride(0); a.gate_sigmoid = gate_sigmoid ? 1 : 0;
+  a.norm_w = f32p(norm_w, "norm_w", vdim);
+  a.eps = (float)eps; a.q_scale = (float)q_scale;
+  a.state = const_cast<float*>(f32p(state, "state"));
+  a.row_state = i32p(row_state, "row_state", T); a.row_back = i32p(row_back, "row_back", T);
+  a.row_fwd = i32p(row_fwd, "row_fwd", T); a.pos = i32p(pos, "positions", T);
+  a.run_rows = run_rows.has_value() ? i32p(*run_rows, "run_rows", 0) : nullptr;
+  a.runs = run_rows.has_value() ? (int)run_rows->numel() : 0;
+  a.out = out.data_ptr();
+  a.T = T; a.H = H; a.rep = H / Hq; a.dim = dim; a.vdim = vdim; a.slots = (int)state.size(0) / 2;
+  rfqmix::launch_gated_linrec(in_f32, a_f32, beta.has_value(), a, stream());
+}
+
+void moe_route_topk(const Tensor& z, const OptT& bias, int64_t top, const Tensor& ids,
+                    const Tensor& weights) {
+  TORCH_CHECK(z.dim() == 2, "moe_route_topk: z [T, E]");
+  const int T = (int)z.size(0), E = (int)z.size(1);
+  TORCH_CHECK(top >= 1 && top <= E, "moe_route_topk: top");
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == at::kInt && ids.is_contiguous() &&
+              ids.numel() == (int64_t)T * top, "moe_route_topk: ids [T, top] int32");
+  rfqmix::launch_moe_route_topk(f32p(z, "z"), optf(bias, "bias", E), T, E, (int)top,
+                                ids.data_ptr<int32_t>(),
+                                const_cast<float*>(f32p(weights, "weights", (int64_t)T * top)),
+                                stream());
+}
+
+void gelu_rows(const Tensor& x, const Tensor& out) {
+  const bool f32 = act_f32(x, "gelu_rows x");
+  TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1 && out.is_cuda() &&
+              out.scalar_type() == x.scalar_type() && rows2d(out, x.size(0), x.size(1)),
+              "gelu_rows: x, out [T, F] of one type");
+  rfqmix::launch_gelu_rows(f32, x.data_ptr(), x.stride(0), out.data_ptr(), out.stride(0),
+                           (int)x.size(0), (int)x.size(1), stream());
+}
+
 }  // namespace
 
 TORCH_LIBRARY(rfq_mix, m) {
@@ -499,6 +706,13 @@ TORCH_LIBRARY(rfq_mix, m) {
   m.def("wkv_recurrence(Tensor r, Tensor k, Tensor v, Tensor zw, Tensor w0, Tensor u, Tensor gate, Tensor norm_w, float eps, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor? run_rows, Tensor(b!) out) -> ()");
   m.def("moe_route_grouped(Tensor z, Tensor correction, int top, int groups, int keep, Tensor(a!) ids, Tensor(b!) weights) -> ()");
   m.def("moe_pair_up(Tensor h, Tensor ids, Tensor w13, Tensor(a!) act) -> ()");
+  m.def("residual_add_norm(Tensor(a!) x, Tensor? y1, Tensor? y2, Tensor? shift, Tensor? w, float eps, float offset, Tensor(b!)? out) -> ()");
+  m.def("rotary_append(Tensor qkv, Tensor pos, Tensor inv_freq, Tensor slots, Tensor(a!) k_cache, Tensor(b!) v_cache, int H, int G, int maps, int dim, int vdim, Tensor(c!) q_out) -> ()");
+  m.def("attn_diff_window(Tensor q, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor gate, Tensor(a!) out, float scale, int window, float lam, float eps, float out_mult) -> ()");
+  m.def("conv_act_heads(Tensor x, Tensor w, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, int n_unit, int dim, float unit_eps, Tensor(b!) out) -> ()");
+  m.def("gated_linear_recurrence(Tensor q, Tensor k, Tensor v, Tensor z, Tensor rate, Tensor zbias, float zsign, Tensor? beta, Tensor gate, bool gate_sigmoid, Tensor norm_w, float eps, float q_scale, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor? run_rows, Tensor(b!) out) -> ()");
+  m.def("moe_route_topk(Tensor z, Tensor? bias, int top, Tensor(a!) ids, Tensor(b!) weights) -> ()");
+  m.def("gelu_rows(Tensor x, Tensor(a!) out) -> ()");
   m.def("moe_pair_down(Tensor act, Tensor ids, Tensor weights, Tensor w2, Tensor? base, Tensor(a!) out) -> ()");
 }
 
@@ -523,4 +737,11 @@ TORCH_LIBRARY_IMPL(rfq_mix, CUDA, m) {
   m.impl("moe_route_grouped", &moe_route_grouped);
   m.impl("moe_pair_up", &moe_pair_up);
   m.impl("moe_pair_down", &moe_pair_down);
+  m.impl("residual_add_norm", &residual_add_norm);
+  m.impl("rotary_append", &rotary_append);
+  m.impl("attn_diff_window", &attn_diff_window);
+  m.impl("conv_act_heads", &conv_act_heads);
+  m.impl("gated_linear_recurrence", &gated_linear_recurrence);
+  m.impl("moe_route_topk", &moe_route_topk);
+  m.impl("gelu_rows", &gelu_rows);
 }

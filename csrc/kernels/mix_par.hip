@@ -1,0 +1,273 @@
+// Row kernels of parallel-sublayer layers and their mixers' pre-processing:
+//
+//   residual_add_norm   x += y1 + y2 + shift (fp32 stream), then h = rms(x) (w + offset) for
+//                       the next layer: one kernel per layer boundary
+//   rotary_append       interleaved-pair rotation of the leading dimensions of every score
+//                       map of q and k; k and v into their pages, q out in fp32
+//   conv_act_heads      causal convolution over time + silu of projection outputs, with the
+//                       last taps - 1 inputs kept per sequence; leading heads made unit vectors
+//   moe_route_topk      largest router logits (+ bias), softmax over the chosen ones
+//   gelu_rows           exact gelu
+//
+// One workgroup per token row (the router: one thread per row).  Norms, angles, the stream,
+// the convolution state and the router are fp32 whatever the activation type is.
+#include "mix_common.h"
+
+namespace rfqmix {
+
+__device__ __forceinline__ float ld_any(const void* p, bool f32, int64_t i) {
+  return f32 ? static_cast<const float*>(p)[i] : ldf(static_cast<const bf16_t*>(p) + i);
+}
+
+// x[t] += y1[t] + y2[t] + shift; out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * (w + offset).
+// y1, y2, shift and (w, out) are each optional; y1 / y2 are fp32 or bf16 (flags).
+template <typename TO>
+__global__ __launch_bounds__(256) void residual_add_norm_kernel(
+    float* __restrict__ x, const void* __restrict__ y1, int64_t y1_stride, bool y1_f32,
+    const void* __restrict__ y2, int64_t y2_stride, bool y2_f32, const float* __restrict__ shift,
+    const float* __restrict__ w, float eps, float offset, TO* __restrict__ out, int d) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  float* xr = x + (int64_t)t * d;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < d; c += blockDim.x) {
+    float v = xr[c];
+    if (y1 != nullptr) v += ld_any(y1, y1_f32, (int64_t)t * y1_stride + c);
+    if (y2 != nullptr) v += ld_any(y2, y2_f32, (int64_t)t * y2_stride + c);
+    if (shift != nullptr) v += shift[c];
+    xr[c] = v;
+    ss += v * v;
+  }
+  if (w == nullptr) return;
+  ss = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(ss / (float)d + eps);
+  // every thread re-reads the entries it wrote itself
+  for (int c = threadIdx.x; c < d; c += blockDim.x)
+    stf(out + (int64_t)t * d + c, xr[c] * r * (w[c] + offset));
+}
+
+// Row t of qkv = q [H][maps][dim] | k [G][maps][dim] | v [G][vdim].  Entries (2i, 2i+1),
+// i < nrot, of every map of q and k turn by the angle pos * inv_freq[i].
+template <typename T>
+__global__ __launch_bounds__(256) void rotary_append_kernel(
+    const T* __restrict__ qkv, int64_t stride, const int32_t* __restrict__ pos,
+    const float* __restrict__ inv_freq, int nrot, const int32_t* __restrict__ slots,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G, int maps, int dim, int vdim,
+    int BS, int64_t pool_slots, float* __restrict__ q_out) {
+  const int t = blockIdx.x;
+  const T* row = qkv + (int64_t)t * stride;
+  const float p = (float)pos[t];
+  const int32_t slot = slots[t];
+  const bool keep = slot >= 0 && slot < pool_slots;
+  const int half = dim / 2 + (dim & 1);              // pairs per map (+ a lone last entry)
+  const int nqp = H * maps * half, nkp = G * maps * half;
+  const int kw = maps * dim;
+  for (int x = threadIdx.x; x < nqp + nkp; x += blockDim.x) {
+    const bool is_q = x < nqp;
+    const int y = is_q ? x : x - nqp;
+    const int hm = y / half, i = y - hm * half;      // (head, map) and pair index
+    const int e = hm * dim + 2 * i;                  // offset inside q or k
+    const T* src = row + (is_q ? 0 : H * kw) + e;
+    const bool pair = 2 * i + 1 < dim;
+    float u = ldf(src), v = pair ? ldf(src + 1) : 0.f;
+    if (i < nrot && pair) {
+      float sn, cs;
+      sincosf(p * inv_freq[i], &sn, &cs);
+      const float a = u * cs - v * sn, b = v * cs + u * sn;
+      u = a;
+      v = b;
+    }
+    if (is_q) {
+      float* o = q_out + (int64_t)t * H * kw + e;
+      o[0] = u;
+      if (pair) o[1] = v;
+    } else if (keep) {
+      const int g = hm / maps, off = e - g * kw;
+      T* o = k_cache + (((int64_t)(slot / BS) * G + g) * BS + slot % BS) * (int64_t)kw + off;
+      stf(o, u);
+      if (pair) stf(o + 1, v);
+    }
+  }
+  if (keep) {
+    const T* vs = row + (int64_t)(H + G) * kw;
+    for (int x = threadIdx.x; x < G * vdim; x += blockDim.x) {
+      const int g = x / vdim, e = x - g * vdim;
+      v_cache[(((int64_t)(slot / BS) * G + g) * BS + slot % BS) * (int64_t)vdim + e] = vs[x];
+    }
+  }
+}
+
+// y[t, c] = silu(sum_j w[c, j] x[t - (taps-1-j), c]); rows before the run come from the
+// sequence's state half, rows before position 0 are zero; the run's last taps - 1 inputs go
+// to the other half.  Then heads [0, n_unit) of `dim` channels become unit vectors.
+// LDS: C floats.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_act_heads_kernel(
+    const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
+    float* __restrict__ state, const int32_t* __restrict__ row_state,
+    const int32_t* __restrict__ row_back, const int32_t* __restrict__ row_fwd,
+    const int32_t* __restrict__ pos, float* __restrict__ out, int C, int taps, int slots,
+    int n_unit, int dim, float unit_eps) {
+  extern __shared__ float ys[];
+  const int t = blockIdx.x;
+  const int code = row_state[t], i = row_back[t], f = row_fwd[t], p = pos[t];
+  const int K = taps - 1;
+  const float* rd = code >= 0 ? state + ((int64_t)((code & 1) * slots + (code >> 1)) * K) * C : nullptr;
+  float* wr = code >= 0 ? state + ((int64_t)((1 - (code & 1)) * slots + (code >> 1)) * K) * C : nullptr;
+  const T* xr = x + (int64_t)t * x_stride;
+  const int n = i + f + 1;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    const float x0 = ldf(xr + c);
+    const float* wc = w + (int64_t)c * taps;
+    float acc = wc[taps - 1] * x0;
+    for (int dl = 1; dl < taps; ++dl) {
+      float src;
+      if (dl <= i) src = ldf(xr - (int64_t)dl * x_stride + c);
+      else if (p - dl >= 0 && rd != nullptr) src = rd[(int64_t)(K + i - dl) * C + c];
+      else continue;
+      acc += wc[taps - 1 - dl] * src;
+    }
+    ys[c] = acc / (1.0f + expf(-acc));
+    if (wr != nullptr) {
+      if (f < K) wr[(int64_t)(K - 1 - f) * C + c] = x0;
+      if (i == 0)
+        for (int e = 0; e < K - n; ++e) wr[(int64_t)e * C + c] = rd[(int64_t)(e + n) * C + c];
+    }
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  float* o = out + (int64_t)t * C;
+  for (int hd = wid; hd < n_unit; hd += nw) {
+    float ss = 0.f;
+    for (int e = lane; e < dim; e += 64) {
+      const float v = ys[hd * dim + e];
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float r = 1.0f / sqrtf(ss + unit_eps);
+    for (int e = lane; e < dim; e += 64) o[hd * dim + e] = ys[hd * dim + e] * r;
+  }
+  for (int c = n_unit * dim + threadIdx.x; c < C; c += blockDim.x) o[c] = ys[c];
+}
+
+// One thread per row: the `top` largest of z + bias (ties to the lower index), weights =
+// softmax over the chosen.  E <= 256.
+__global__ __launch_bounds__(64) void moe_route_topk_kernel(
+    const float* __restrict__ z, const float* __restrict__ bias, int T_, int E, int top,
+    int32_t* __restrict__ ids, float* __restrict__ weights) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T_) return;
+  const float* zr = z + (int64_t)t * E;
+  int32_t* id = ids + (int64_t)t * top;
+  float* wt = weights + (int64_t)t * top;
+  float prev = __builtin_huge_valf();
+  int prev_i = -1;
+  float mx = 0.f;
+  for (int k = 0; k < top; ++k) {
+    // the largest entry after (prev, prev_i) in the order (value descending, index ascending)
+    float best = -__builtin_huge_valf();
+    int bi = -1;
+    for (int e = 0; e < E; ++e) {
+      const float v = zr[e] + (bias != nullptr ? bias[e] : 0.f);
+      const bool after = v < prev || (v == prev && e > prev_i);
+      if (after && (bi < 0 || v > best)) {
+        best = v;
+        bi = e;
+      }
+    }
+    if (bi < 0) {                       // non-finite logits: keep the indices valid
+      bi = k < E ? k : 0;
+      best = -__builtin_huge_valf();
+    }
+    id[k] = bi;
+    wt[k] = best;
+    if (k == 0) mx = best;
+    prev = best;
+    prev_i = bi;
+  }
+  float sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    const float e = expf(wt[k] - mx);
+    wt[k] = e;
+    sum += e;
+  }
+  for (int k = 0; k < top; ++k) wt[k] /= sum;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_rows_kernel(const T* __restrict__ x, int64_t x_stride,
+                                                        T* __restrict__ out, int64_t o_stride,
+                                                        int F) {
+  const int t = blockIdx.x;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < F; c += gridDim.y * blockDim.x) {
+    const float v = ldf(x + (int64_t)t * x_stride + c);
+    stf(out + (int64_t)t * o_stride + c, 0.5f * v * (1.0f + erff(v * 0.70710678118654752f)));
+  }
+}
+
+// ------------------------------------------------------------------ launchers
+void launch_residual_add_norm(bool out_f32, float* x, const void* y1, int64_t y1s, bool y1f,
+                              const void* y2, int64_t y2s, bool y2f, const float* shift,
+                              const float* w, float eps, float offset, void* out, int T_, int d,
+                              hipStream_t s) {
+  if (T_ == 0) return;
+  if (out_f32)
+    hipLaunchKernelGGL(residual_add_norm_kernel<float>, dim3(T_), dim3(256), 0, s, x, y1, y1s, y1f,
+                       y2, y2s, y2f, shift, w, eps, offset, (float*)out, d);
+  else
+    hipLaunchKernelGGL(residual_add_norm_kernel<bf16_t>, dim3(T_), dim3(256), 0, s, x, y1, y1s,
+                       y1f, y2, y2s, y2f, shift, w, eps, offset, (bf16_t*)out, d);
+}
+
+void launch_rotary_append(bool f32, const void* qkv, int64_t stride, const int32_t* pos,
+                          const float* inv_freq, int nrot, const int32_t* slots, void* k_cache,
+                          void* v_cache, int T_, int H, int G, int maps, int dim, int vdim, int BS,
+                          int64_t pool_slots, float* q_out, hipStream_t s) {
+  if (T_ == 0) return;
+  if (f32)
+    hipLaunchKernelGGL(rotary_append_kernel<float>, dim3(T_), dim3(256), 0, s, (const float*)qkv,
+                       stride, pos, inv_freq, nrot, slots, (float*)k_cache, (float*)v_cache, H, G,
+                       maps, dim, vdim, BS, pool_slots, q_out);
+  else
+    hipLaunchKernelGGL(rotary_append_kernel<bf16_t>, dim3(T_), dim3(256), 0, s, (const bf16_t*)qkv,
+                       stride, pos, inv_freq, nrot, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, H, G,
+                       maps, dim, vdim, BS, pool_slots, q_out);
+}
+
+void launch_conv_act_heads(bool f32, const void* x, int64_t stride, const float* w, float* state,
+                           const int32_t* row_state, const int32_t* row_back,
+                           const int32_t* row_fwd, const int32_t* pos, float* out, int T_, int C,
+                           int taps, int slots, int n_unit, int dim, float unit_eps,
+                           hipStream_t s) {
+  if (T_ == 0) return;
+  const size_t lds = (size_t)C * sizeof(float);          // checked <= 64 KB by the caller
+  if (f32)
+    hipLaunchKernelGGL(conv_act_heads_kernel<float>, dim3(T_), dim3(256), lds, s, (const float*)x,
+                       stride, w, state, row_state, row_back, row_fwd, pos, out, C, taps, slots,
+                       n_unit, dim, unit_eps);
+  else
+    hipLaunchKernelGGL(conv_act_heads_kernel<bf16_t>, dim3(T_), dim3(256), lds, s,
+                       (const bf16_t*)x, stride, w, state, row_state, row_back, row_fwd, pos, out,
+                       C, taps, slots, n_unit, dim, unit_eps);
+}
+
+void launch_moe_route_topk(const float* z, const float* bias, int T_, int E, int top, int32_t* ids,
+                           float* weights, hipStream_t s) {
+  if (T_ == 0) return;
+  hipLaunchKernelGGL(moe_route_topk_kernel, dim3((T_ + 63) / 64), dim3(64), 0, s, z, bias, T_, E,
+                     top, ids, weights);
+}
+
+void launch_gelu_rows(bool f32, const void* x, int64_t xs, void* out, int64_t os, int T_, int F,
+                      hipStream_t s) {
+  if (T_ == 0) return;
+  const dim3 grid(T_, (unsigned)((F + 1023) / 1024 > 0 ? (F + 1023) / 1024 : 1));
+  if (f32)
+    hipLaunchKernelGGL(gelu_rows_kernel<float>, grid, dim3(256), 0, s, (const float*)x, xs,
+                       (float*)out, os, F);
+  else
+    hipLaunchKernelGGL(gelu_rows_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)x, xs,
+                       (bf16_t*)out, os, F);
+}
+
+}  // namespace rfqmix

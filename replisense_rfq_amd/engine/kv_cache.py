@@ -51,19 +51,24 @@ class KVCache:
 class LayeredKVCache:
     """Pools of a layer-list model, all indexed by the block ids of the one block manager.
 
-    Per layer, by the kind of its mixer:
+    Pools and state are held per layer RUN (``cfg.runs``: a layer that a loop runs several
+    times has pages and state of its own in every pass; without a loop a run is a layer).
+    Per run, by the kind of its mixer:
       attention          one K and one V pool with the layer's own head count and sizes
                          (``[num_blocks, G, block, dim]`` / ``[..., vdim]``);
       latent_attention   one pool ``[num_blocks, 1, block, kv_rank]`` of cached latents that
                          serves as keys and as values; a layer that reads another layer's
                          latent holds that layer's pool (the same tensor);
-      wkv                no pages.
+      diff_attention     K pool ``[num_blocks, G, block, 2 dim]`` (both score maps of a
+                         key head side by side) and V pool ``[num_blocks, G, block, vdim]``;
+      wkv, gla, channel_delta   no pages.
     Per-sequence state lives in slots; a sequence owns one while it runs (native core).  Every
     state pool is double buffered: a step reads half ``gen & 1`` of the slot and writes the
     other, so rows of one launch never read what the launch writes.  ``state``: the input
     convolutions' last inputs ``[L, 2 sublayers, 2 * slots, taps - 1, d]`` fp32;
     ``layer_state[i]``: name -> ``[2 * slots, ...]`` fp32 for what ``cfg.state_shapes(i)``
-    lists (a wkv layer's matrices and its previous input row)."""
+    lists (a wkv layer's matrices and its previous input row; a gla or channel_delta
+    layer's matrices, and the convolutions' last inputs)."""
 
     def __init__(self, cfg, num_blocks: int, device, num_slots: int, block_size: int = 32,
                  dtype=torch.bfloat16, prefix_cache: bool = False):
@@ -73,12 +78,18 @@ class LayeredKVCache:
         self.num_slots = num_slots
         mk = torch.zeros if torch.device(device).type != "cuda" else torch.empty
         self.k, self.v = [], []
-        for ly in cfg.layers:
-            m = ly.mixer
+        runs = tuple(getattr(cfg, "runs", range(cfg.n_layers)))
+        for li in runs:
+            m = cfg.layers[li].mixer
             if m.kind == "attention":
                 self.k.append(mk((num_blocks, m.kv_heads, block_size, m.dim), dtype=dtype, device=device))
                 self.v.append(mk((num_blocks, m.kv_heads, block_size, m.vdim), dtype=dtype, device=device))
+            elif m.kind == "diff_attention":
+                self.k.append(mk((num_blocks, m.kv_heads, block_size, 2 * m.dim), dtype=dtype, device=device))
+                self.v.append(mk((num_blocks, m.kv_heads, block_size, m.vdim), dtype=dtype, device=device))
             elif m.kind == "latent_attention":
+                if m.kv_from >= 0 and len(runs) != cfg.n_layers:
+                    raise ValueError("a layer that reads another layer's latent cannot be looped")
                 pool = self.k[m.kv_from] if m.kv_from >= 0 else \
                     mk((num_blocks, 1, block_size, m.kv_rank), dtype=dtype, device=device)
                 self.k.append(pool)
@@ -91,8 +102,8 @@ class LayeredKVCache:
                                  dtype=torch.float32, device=device)
         self.layer_state = [{name: torch.zeros((2 * num_slots,) + tuple(shape), dtype=torch.float32,
                                                device=device)
-                             for name, shape in cfg.state_shapes(i).items()}
-                            for i in range(cfg.n_layers)]
+                             for name, shape in cfg.state_shapes(li).items()}
+                            for li in runs]
         self.scratch_block = num_blocks - 1
         self.prefix_cache = False            # a cached page carries no per-sequence state
         self.core = None

@@ -12,4 +12,8 @@ def layered_model_class(architecture: str):
         from .numalorn import NumalornLM
 
         return NumalornLM
+    if architecture == "Bilolix":
+        from .bilolix import BilolixLM
+
+        return BilolixLM
     raise KeyError(f"no model class for architecture {architecture!r}")

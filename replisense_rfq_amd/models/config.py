@@ -96,7 +96,16 @@ class MixerSpec:
     ``latent_attention``: queries through a ``q_rank`` latent, keys and values are per-head
     up-projections of one cached ``kv_rank`` latent per token; ``kv_from`` >= 0 names the
     layer whose cached latent this layer reads instead of projecting its own.
-    ``wkv``: ``heads`` recurrent heads with a ``dim`` x ``dim`` state each (no cache pages)."""
+    ``wkv``: ``heads`` recurrent heads with a ``dim`` x ``dim`` state each (no cache pages).
+    ``diff_attention``: every head holds two score maps (queries and keys of width
+    2 * ``dim``, laid out [map 1 | map 2]) over the same values; rotary positions on the
+    first ``rot_dims`` dimensions of each map (``rot_base``), position i sees the ``window``
+    positions up to itself (0 = plain causal), the second map's output is subtracted with a
+    learned weight whose constant part is ``diff``.
+    ``gla``: ``heads`` recurrent heads with a ``dim`` x ``vdim`` state and a decay per key
+    channel, sigmoid(z)^(1 / ``tau``).
+    ``channel_delta``: the gated delta rule on such states; queries and keys have
+    ``kv_heads`` heads, and q, k, v pass a causal convolution of ``conv`` taps."""
     kind: str = "attention"
     heads: int = 4
     kv_heads: int = 2
@@ -107,6 +116,12 @@ class MixerSpec:
     q_rank: int = 0
     kv_rank: int = 0
     kv_from: int = -1
+    window: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    diff: float = 0.0
+    tau: float = 1.0
+    conv: int = 0
 
     @property
     def group(self) -> int:
@@ -118,7 +133,9 @@ class MlpSpec:
     """``dense``: clamped GLU of width ``ff``.  ``moe``: ``experts`` SwiGLU experts of width
     ``ff``, ``top`` per token, chosen among the ``keep`` best of ``groups`` equal groups of
     neighbouring experts (groups = 0: no limit), plus a shared expert of width
-    ``shared_ff`` (0: none)."""
+    ``shared_ff`` (0: none); ``router`` = ``softmax_top``: the ``top`` largest router logits
+    (with a bias), weighted by the softmax over the chosen logits only.  ``gelu``: up
+    projection, exact gelu, down projection."""
     kind: str = "dense"
     ff: int = 256
     limit: float = 7.0
@@ -127,6 +144,7 @@ class MlpSpec:
     groups: int = 0
     keep: int = 0
     shared_ff: int = 0
+    router: str = "grouped_sigmoid"
 
 
 @dataclass(frozen=True)
@@ -153,10 +171,32 @@ class LayeredConfig:
     residual_mult: float = 1.0      # Numalorn: x += residual_mult * norm(sublayer(x))
     logit_softcap: float = 0.0      # > 0: logits <- cap * tanh(logits / cap)
     decay_rank: int = 16            # wkv layers of seeded models (a checkpoint's shapes decide)
+    # layers loop[0] .. loop[1]-1 run loop[2] times in a row on the same weights; every pass
+    # has cache pages and state of its own
+    loop: tuple = (0, 0, 1)
+    gate_rank: int = 16             # channel_delta layers of seeded models (output gate's inner size)
 
     @property
     def n_layers(self) -> int:
         return len(self.layers)
+
+    @property
+    def runs(self) -> tuple:
+        """Layer index of every layer run of a forward pass, in order (a looped layer counts
+        once per pass).  Caches and state are held per run."""
+        a, b, times = self.loop
+        n = len(self.layers)
+        if b <= a or times == 1:
+            return tuple(range(n))
+        return tuple(range(a)) + tuple(range(a, b)) * times + tuple(range(b, n))
+
+    @property
+    def pass_starts(self) -> dict:
+        """Run index at which pass t of the loop starts -> t (empty without a loop)."""
+        a, b, times = self.loop
+        if b <= a:
+            return {}
+        return {a + t * (b - a): t for t in range(times)}
 
     @property
     def is_moe(self) -> bool:
@@ -174,21 +214,32 @@ class LayeredConfig:
             elif m.kind == "latent_attention":
                 n += d * m.q_rank + m.q_rank * m.heads * m.dim + m.heads * m.vdim * d
                 n += m.kv_rank * m.heads * (m.dim + m.vdim) + (d * m.kv_rank if m.kv_from < 0 else 0)
+            elif m.kind == "diff_attention":
+                n += d * (2 * m.dim * (m.heads + m.kv_heads) + m.kv_heads * m.vdim + m.heads)
+                n += m.heads * m.vdim * d
+            elif m.kind == "gla":
+                n += 2 * d * m.heads * (m.dim + m.vdim) + m.heads * m.vdim * d
+                n += self.decay_rank * (d + m.heads * m.dim)
+            elif m.kind == "channel_delta":
+                n += d * (2 * m.kv_heads * m.dim + m.heads * m.vdim + m.heads) + m.heads * m.vdim * d
+                n += self.decay_rank * (d + m.heads * m.dim) + self.gate_rank * (d + m.heads * m.vdim)
             else:
                 n += 5 * d * m.heads * m.dim + 2 * d * self.decay_rank
             f = ly.mlp
             if f is not None and f.kind == "moe":
                 n += 3 * d * (f.ff * f.experts + f.shared_ff) + d * f.experts
             elif f is not None:
-                n += 3 * d * f.ff
+                n += (2 if f.kind == "gelu" else 3) * d * f.ff
         return n + 2 * self.vocab_size * d + d
 
     def kv_bytes_per_token(self, tp: int = 1, dtype_bytes: int = 2) -> int:
         n = 0
-        for ly in self.layers:
-            m = ly.mixer
+        for li in self.runs:
+            m = self.layers[li].mixer
             if m.kind == "attention":
                 n += m.kv_heads * (m.dim + m.vdim)
+            elif m.kind == "diff_attention":
+                n += m.kv_heads * (2 * m.dim + m.vdim)
             elif m.kind == "latent_attention" and m.kv_from < 0:
                 n += m.kv_rank
         return max(1, n) * dtype_bytes
@@ -199,6 +250,11 @@ class LayeredConfig:
         m = self.layers[li].mixer
         if m.kind == "wkv":
             return {"wkv": (m.heads, m.dim, m.dim), "prev": (self.hidden,)}
+        if m.kind == "gla":
+            return {"S": (m.heads, m.dim, m.vdim)}
+        if m.kind == "channel_delta":
+            return {"S": (m.heads, m.dim, m.vdim),
+                    "conv": (max(0, m.conv - 1), 2 * m.kv_heads * m.dim + m.heads * m.vdim)}
         return {}
 
     def to_dict(self):
@@ -278,6 +334,81 @@ def numalorn_from_json(d: dict, name: str | None = None) -> LayeredConfig:
                          logit_softcap=float(d.get("logit_softcap") or 0.0))
 
 
+def bilolix_from_json(d: dict, name: str | None = None) -> LayeredConfig:
+    """config.json of a Bilolix checkpoint: vocab, width, norm.eps, ``loop`` (start, stop,
+    times; optional) and ``layers``: type ``attention`` (heads, kv_heads, dim, vdim, scale,
+    diff, mask.size, rot.dims, rot.base), ``gla`` (heads, dim, vdim, tau) or ``channel_delta``
+    (heads, kv_heads, dim, vdim, conv), each with an ``mlp`` of kind ``dense`` (ff), ``moe``
+    (expert.ff, router.experts, router.top) or null."""
+    layers = []
+    for i, ly in enumerate(d["layers"]):
+        m, kind = ly["mixer"], ly["type"]
+        if kind == "attention":
+            rot = m.get("rot") or {}
+            mixer = MixerSpec("diff_attention", int(m["heads"]), int(m["kv_heads"]), int(m["dim"]),
+                              int(m["vdim"]), float(m["scale"]),
+                              window=int((m.get("mask") or {}).get("size", 0)),
+                              rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)),
+                              diff=float(m["diff"]))
+            if mixer.rot_dims % 2 or mixer.rot_dims > mixer.dim:
+                raise ValueError(f"layer {i}: rot.dims must be even and at most dim")
+        elif kind == "gla":
+            mixer = MixerSpec("gla", int(m["heads"]), int(m["heads"]), int(m["dim"]), int(m["vdim"]),
+                              float(m["dim"]) ** -0.5, tau=float(m["tau"]))
+        elif kind == "channel_delta":
+            mixer = MixerSpec("channel_delta", int(m["heads"]), int(m["kv_heads"]), int(m["dim"]),
+                              int(m["vdim"]), float(m["dim"]) ** -0.5, conv=int(m["conv"]))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        if mixer.heads % mixer.kv_heads:
+            raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+        f = ly.get("mlp")
+        mlp = None
+        if f is not None and f.get("kind") == "dense":
+            mlp = MlpSpec("gelu", int(f["ff"]), 0.0)
+        elif f is not None and f.get("kind") == "moe":
+            r = f["router"]
+            if not 0 < int(r["top"]) <= int(r["experts"]):
+                raise ValueError(f"layer {i}: top must be between 1 and the number of experts")
+            mlp = MlpSpec("moe", int(f["expert"]["ff"]), 0.0, int(r["experts"]), int(r["top"]),
+                          router="softmax_top")
+        elif f is not None:
+            raise ValueError(f"layer {i}: unknown feed-forward kind {f.get('kind')!r}")
+        layers.append(LayerSpec(mixer, mlp))
+    lp = d.get("loop") or {}
+    loop = (int(lp.get("start", 0)), int(lp.get("stop", 0)), int(lp.get("times", 1)))
+    if loop[1] > loop[0] and not (0 <= loop[0] and loop[1] <= len(layers) and loop[2] >= 1):
+        raise ValueError("loop: start .. stop must lie inside the layers, times >= 1")
+    return LayeredConfig(name=name or d["architecture"].lower(), architecture=d["architecture"],
+                         vocab_size=int(d["vocab"]), hidden=int(d["width"]), layers=tuple(layers),
+                         rms_eps=float(d["norm"]["eps"]), canon_taps=0,
+                         max_position=int(d.get("max_position", 8192)), loop=loop)
+
+
+def bilolix_layers(order, heads, kv_heads, dim, vdim, ff, experts=0, top=0, expert_ff=0,
+                   window=0, rot_dims=None, rot_base=10000.0, diff=0.5, tau=16.0, conv=4,
+                   rec_heads=None, rec_kv_heads=None):
+    """Layers of the kinds named in ``order`` ("a" differential attention, "g" gla, "c"
+    channel_delta); with experts, every second layer's feed-forward is a mixture."""
+    rh = rec_heads or heads
+    rk = rec_kv_heads or rh
+    out = []
+    for i, c in enumerate(order):
+        if c == "a":
+            m = MixerSpec("diff_attention", heads, kv_heads, dim, vdim, dim ** -0.5, window=window,
+                          rot_dims=dim if rot_dims is None else rot_dims, rot_base=rot_base, diff=diff)
+        elif c == "g":
+            m = MixerSpec("gla", rh, rh, dim, vdim, dim ** -0.5, tau=tau)
+        else:
+            m = MixerSpec("channel_delta", rh, rk, dim, vdim, dim ** -0.5, conv=conv)
+        if experts and i % 2 == 1:
+            f = MlpSpec("moe", expert_ff, 0.0, experts, top, router="softmax_top")
+        else:
+            f = MlpSpec("gelu", ff, 0.0) if ff else None
+        out.append(LayerSpec(m, f))
+    return tuple(out)
+
+
 def numalorn_layers(n, width_heads, dim, vdim, q_rank, kv_rank, wkv_heads, ff, experts, top,
                     groups, keep, shared_ff, share_every=2, wkv_dim=64):
     """n layers alternating latent attention and wkv; of every ``share_every`` attention
@@ -308,10 +439,19 @@ LIVISUN_8B = LayeredConfig("livisun-8b", vocab_size=128256, hidden=4096, embed_s
 TINY_NUMALORN = LayeredConfig("tiny-numalorn", architecture="Numalorn", vocab_size=320, hidden=128,
                               canon_taps=0, residual_mult=0.5, logit_softcap=20.0, decay_rank=8,
                               layers=numalorn_layers(4, 4, 32, 16, 48, 64, 2, 64, 6, 2, 3, 2, 96))
-CONFIGS.update({c.name: c for c in (TINY_LIVISUN, LIVISUN_8B, TINY_NUMALORN)})
+# attention, gla and channel_delta layers; layers 1 .. 2 run twice; sizes that differ from
+# each other wherever the design allows (dim != vdim, rot_dims < dim, kv_heads < heads)
+TINY_BILOLIX = LayeredConfig("tiny-bilolix", architecture="Bilolix", vocab_size=352, hidden=96,
+                             canon_taps=0, decay_rank=8, gate_rank=12, loop=(1, 3, 2),
+                             layers=bilolix_layers("agca", 6, 2, 16, 24, 160, experts=5, top=3,
+                                                   expert_ff=40, window=21, rot_dims=8,
+                                                   rot_base=5000.0, diff=0.7, tau=8.0, conv=3,
+                                                   rec_heads=4, rec_kv_heads=2))
+CONFIGS.update({c.name: c for c in (TINY_LIVISUN, LIVISUN_8B, TINY_NUMALORN, TINY_BILOLIX)})
 
 # config.json "architecture" -> reader
-ARCHITECTURES = {"Livisun": LayeredConfig.from_json, "Numalorn": numalorn_from_json}
+ARCHITECTURES = {"Livisun": LayeredConfig.from_json, "Numalorn": numalorn_from_json,
+                 "Bilolix": bilolix_from_json}
 
 
 def load_config(path: str):

@@ -295,6 +295,8 @@ def load_layered_safetensors(path: str, cfg, device, dtype=torch.bfloat16) -> di
     ck = _LazyCheckpoint(files)
     if cfg.architecture == "Numalorn":
         return _numalorn_assemble(ck.full, lambda k: k in ck, cfg, device, dtype)
+    if cfg.architecture == "Bilolix":
+        return _bilolix_assemble(ck.full, lambda k: k in ck, cfg, device, dtype)
     w = {"embed": ck.full("embed").to(dtype).to(device), "lm_head": ck.full("head").to(dtype).to(device),
          "final_norm": ck.full("final.norm").float().to(device), "vocab_start": 0, "layers": []}
     for i, ly in enumerate(cfg.layers):
@@ -506,5 +508,205 @@ def init_numalorn_weights(cfg, device, dtype=torch.bfloat16, seed: int = 0,
 
 def numalorn_from_full(full: dict, cfg, device, dtype=torch.bfloat16) -> dict:
     w = _numalorn_assemble(lambda k: full[k], lambda k: k in full, cfg, device, dtype)
+    w["full"] = full
+    return w
+
+
+# --------------------------------------------------------------------------
+# Bilolix.  Checkpoint names:
+#   embed, head [V, d]; final.norm [d]; loop.step [times, d]; l<i>.norm1 [d] (stored around zero)
+#   attention: l<i>.mix.q [H*2*dim, d]  .k [G*2*dim, d]  .v [G*vdim, d]  .g [H, d]  .o [d, H*vdim]
+#     .lq1 | .lk1 | .lq2 | .lk2 [dim]
+#   gla: l<i>.mix.q | .k [H*dim, d]  .v | .g [H*vdim, d]  .a1 [rank, d]  .a2 [H*dim, rank]
+#     .a2.b [H*dim]  .norm [vdim]  .o [d, H*vdim]
+#   channel_delta: l<i>.mix.q | .k [G*dim, d]  .v [H*vdim, d]  .q.conv | .k.conv | .v.conv
+#     [channels, taps]  .b [H, d]  .A_log [H]  .a1 [rank, d]  .a2 [H*dim, rank]  .dt_bias [H*dim]
+#     .g1 [grank, d]  .g2 [H*vdim, grank]  .norm [vdim]  .o [d, H*vdim]
+#   dense: l<i>.mlp.up [F, d]  .down [d, F]
+#   moe: l<i>.mlp.router [E, d]  .router.b [E]  .e<j>.gate | up [F, d]  .e<j>.down [d, F]
+# Loaded layout per layer: attention "qkv" = q | k | v rows; the recurrent mixers' input
+# projections are ONE matrix "proj" whose row segments (each padded with zero rows to a
+# multiple of 8, so that every column slice of the product starts 16-byte aligned) are listed
+# in "seg": name -> (first column, width); inner ranks come from the tensors' shapes; the
+# attention's lambda = exp(lq1.lk1) - exp(lq2.lk2) + diff is one float ("lam"); the delta
+# rule's rate exp(A_log) and the gla rate 1 / tau are "rate" [H] fp32; norm weights, biases
+# and convolution taps in fp32.
+SEG_ALIGN = 8
+
+
+def _stack_segments(parts, d, dtype):
+    """[(name, tensor [n, d], pad)] -> (matrix of the segments in order, {name: (first row,
+    n)}); after a segment with ``pad`` zero rows bring the next one to a multiple of
+    SEG_ALIGN (segments that only this package's kernels read need none)."""
+    rows, seg, at = [], {}, 0
+    for name, t, pad in parts:
+        n = t.shape[0]
+        seg[name] = (at, n)
+        rows.append(t.to(dtype))
+        at += n
+        if pad and at % SEG_ALIGN:
+            z = (-at) % SEG_ALIGN
+            rows.append(torch.zeros((z, d), dtype=dtype, device=t.device))
+            at += z
+    return torch.cat(rows, 0).contiguous(), seg
+
+
+def _bilolix_assemble(get, has, cfg, device, dtype) -> dict:
+    import math
+
+    d = cfg.hidden
+
+    def mat(name, rows, cols):
+        t = get(name)
+        if tuple(t.shape) != (rows, cols):
+            raise ValueError(f"tensor {name}: shape {tuple(t.shape)}, expected {(rows, cols)}")
+        return t.to(dtype)
+
+    def lowrank(name, cols):
+        t = get(name)
+        if t.dim() != 2 or t.shape[1] != cols:
+            raise ValueError(f"tensor {name}: shape {tuple(t.shape)}, expected (rank, {cols})")
+        return t.to(dtype)
+
+    def vec(name, *shape):
+        t = get(name)
+        if tuple(t.shape) != tuple(shape):
+            raise ValueError(f"tensor {name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+        return t.float().contiguous().to(device)
+
+    V = cfg.vocab_size
+    w = {"embed": mat("embed", V, d).to(device), "lm_head": mat("head", V, d).to(device),
+         "final_norm": vec("final.norm", d), "vocab_start": 0, "layers": []}
+    a, b, times = cfg.loop
+    if b > a:
+        w["loop_step"] = vec("loop.step", times, d)
+    for i, ly in enumerate(cfg.layers):
+        p, m, lw = f"l{i}.mix.", ly.mixer, LayerWeights()
+        lw["norm1"] = vec(f"l{i}.norm1", d)
+        H, G, dim, vd = m.heads, m.kv_heads, m.dim, m.vdim
+        if m.kind == "diff_attention":
+            lw["qkv"] = torch.cat([mat(p + "q", H * 2 * dim, d), mat(p + "k", G * 2 * dim, d),
+                                   mat(p + "v", G * vd, d)], 0).contiguous().to(device)
+            lw["g"] = mat(p + "g", H, d).contiguous().to(device)
+            lv = [vec(p + n, dim).double().cpu() for n in ("lq1", "lk1", "lq2", "lk2")]
+            lw["lam"] = math.exp(float((lv[0] * lv[1]).sum())) - math.exp(float((lv[2] * lv[3]).sum())) \
+                + m.diff
+        elif m.kind == "gla":
+            a1 = lowrank(p + "a1", d)
+            proj, seg = _stack_segments([("q", mat(p + "q", H * dim, d), 0), ("k", mat(p + "k", H * dim, d), 0),
+                                         ("v", mat(p + "v", H * vd, d), 0), ("g", mat(p + "g", H * vd, d), 1),
+                                         ("a1", a1, 1)], d, dtype)
+            lw["proj"], lw["seg"] = proj.to(device), seg
+            lw["a2"] = mat(p + "a2", H * dim, a1.shape[0]).contiguous().to(device)
+            lw["zbias"] = vec(p + "a2.b", H * dim)
+            lw["rate"] = torch.full((H,), 1.0 / m.tau, dtype=torch.float32, device=device)
+            lw["gn"] = vec(p + "norm", vd)
+        elif m.kind == "channel_delta":
+            a1, g1 = lowrank(p + "a1", d), lowrank(p + "g1", d)
+            proj, seg = _stack_segments([("q", mat(p + "q", G * dim, d), 0), ("k", mat(p + "k", G * dim, d), 0),
+                                         ("v", mat(p + "v", H * vd, d), 0), ("b", mat(p + "b", H, d), 1),
+                                         ("a1", a1, 1), ("g1", g1, 1)], d, dtype)
+            lw["proj"], lw["seg"] = proj.to(device), seg
+            taps = m.conv
+            lw["conv_w"] = torch.cat([vec(p + "q.conv", G * dim, taps), vec(p + "k.conv", G * dim, taps),
+                                      vec(p + "v.conv", H * vd, taps)], 0).contiguous()
+            lw["a2"] = mat(p + "a2", H * dim, a1.shape[0]).contiguous().to(device)
+            lw["zbias"] = vec(p + "dt_bias", H * dim)
+            lw["rate"] = torch.exp(vec(p + "A_log", H).double()).float()
+            lw["g2"] = mat(p + "g2", H * vd, g1.shape[0]).contiguous().to(device)
+            lw["gn"] = vec(p + "norm", vd)
+        else:
+            raise ValueError(f"layer {i}: no weights known for mixer {m.kind!r}")
+        lw["o"] = mat(p + "o", d, H * vd).contiguous().to(device)
+        f, q = ly.mlp, f"l{i}.mlp."
+        if f is not None and f.kind == "moe":
+            lw["router"] = mat(q + "router", f.experts, d).contiguous().to(device)
+            lw["router_b"] = vec(q + "router.b", f.experts)
+            lw["w13"] = torch.stack([torch.cat([mat(f"{q}e{e}.gate", f.ff, d), mat(f"{q}e{e}.up", f.ff, d)], 0)
+                                     for e in range(f.experts)]).contiguous().to(device)
+            lw["w2e"] = torch.stack([mat(f"{q}e{e}.down", d, f.ff) for e in range(f.experts)]) \
+                .contiguous().to(device)
+        elif f is not None:
+            lw["up"] = mat(q + "up", f.ff, d).contiguous().to(device)
+            lw["down"] = mat(q + "down", d, f.ff).contiguous().to(device)
+        w["layers"].append(lw)
+    return w
+
+
+def init_bilolix_weights(cfg, device, dtype=torch.bfloat16, seed: int = 0,
+                         keep_full: bool = True) -> dict:
+    """Seeded random Bilolix weights under the checkpoint's names (tests and benchmarks):
+    projections scaled so that activations stay O(1); lambda vectors, decay biases, step
+    vectors, router biases and zero-centred norm weights away from their neutral values so
+    that each shows in the logits.  ``keep_full`` False (benchmark sizes): drawn on the device,
+    the name -> tensor dict is not kept."""
+    d, full = cfg.hidden, {}
+
+    def rnd(name, shape, std, mean=0.0):
+        if keep_full:
+            t = _randn(shape, std, (seed, name), "cpu", torch.float32) + mean
+            full[name] = t.to(torch.bfloat16).float()
+        else:
+            full[name] = (_randn(shape, std, (seed, name), device, torch.float32) + mean).to(torch.bfloat16)
+        return full[name]
+
+    rnd("embed", (cfg.vocab_size, d), 1.0)
+    rnd("head", (cfg.vocab_size, d), 2.0 * d ** -0.5)
+    rnd("final.norm", (d,), 0.2)
+    if cfg.loop[1] > cfg.loop[0]:
+        rnd("loop.step", (cfg.loop[2], d), 0.5)
+    for i, ly in enumerate(cfg.layers):
+        p, m = f"l{i}.mix.", ly.mixer
+        H, G, dim, vd = m.heads, m.kv_heads, m.dim, m.vdim
+        rnd(f"l{i}.norm1", (d,), 0.2)
+        if m.kind == "diff_attention":
+            rnd(p + "q", (H * 2 * dim, d), 2.0 * d ** -0.5)
+            rnd(p + "k", (G * 2 * dim, d), 2.0 * d ** -0.5)
+            rnd(p + "v", (G * vd, d), d ** -0.5)
+            rnd(p + "g", (H, d), 2.0 * d ** -0.5)
+            for n in ("lq1", "lk1", "lq2", "lk2"):
+                rnd(p + n, (dim,), 0.5 * dim ** -0.5)
+        elif m.kind == "gla":
+            rnd(p + "q", (H * dim, d), 2.0 * d ** -0.5)
+            rnd(p + "k", (H * dim, d), d ** -0.5)
+            rnd(p + "v", (H * vd, d), d ** -0.5)
+            rnd(p + "g", (H * vd, d), 2.0 * d ** -0.5)
+            rnd(p + "a1", (cfg.decay_rank, d), d ** -0.5)
+            rnd(p + "a2", (H * dim, cfg.decay_rank), 2.0 * cfg.decay_rank ** -0.5)
+            rnd(p + "a2.b", (H * dim,), 1.0, 2.0)
+            rnd(p + "norm", (vd,), 0.1, 1.0)
+        else:
+            rnd(p + "q", (G * dim, d), 2.0 * d ** -0.5)
+            rnd(p + "k", (G * dim, d), 2.0 * d ** -0.5)
+            rnd(p + "v", (H * vd, d), 2.0 * d ** -0.5)
+            for n, c in (("q", G * dim), ("k", G * dim), ("v", H * vd)):
+                rnd(p + n + ".conv", (c, m.conv), 0.5)
+            rnd(p + "b", (H, d), 2.0 * d ** -0.5)
+            rnd(p + "A_log", (H,), 0.5, -1.0)
+            rnd(p + "a1", (cfg.decay_rank, d), d ** -0.5)
+            rnd(p + "a2", (H * dim, cfg.decay_rank), 2.0 * cfg.decay_rank ** -0.5)
+            rnd(p + "dt_bias", (H * dim,), 1.0, -1.0)
+            rnd(p + "g1", (cfg.gate_rank, d), d ** -0.5)
+            rnd(p + "g2", (H * vd, cfg.gate_rank), 2.0 * cfg.gate_rank ** -0.5)
+            rnd(p + "norm", (vd,), 0.1, 1.0)
+        rnd(p + "o", (d, H * vd), (H * vd) ** -0.5)
+        f, q = ly.mlp, f"l{i}.mlp."
+        if f is not None and f.kind == "moe":
+            rnd(q + "router", (f.experts, d), 2.0 * d ** -0.5)
+            rnd(q + "router.b", (f.experts,), 0.5)
+            for e in range(f.experts):
+                rnd(f"{q}e{e}.gate", (f.ff, d), d ** -0.5)
+                rnd(f"{q}e{e}.up", (f.ff, d), d ** -0.5)
+                rnd(f"{q}e{e}.down", (d, f.ff), f.ff ** -0.5)
+        elif f is not None:
+            rnd(q + "up", (f.ff, d), d ** -0.5)
+            rnd(q + "down", (d, f.ff), f.ff ** -0.5)
+    if not keep_full:
+        return _bilolix_assemble(lambda k: full.pop(k), lambda k: k in full, cfg, device, dtype)
+    return bilolix_from_full(full, cfg, device, dtype)
+
+
+def bilolix_from_full(full: dict, cfg, device, dtype=torch.bfloat16) -> dict:
+    w = _bilolix_assemble(lambda k: full[k], lambda k: k in full, cfg, device, dtype)
     w["full"] = full
     return w

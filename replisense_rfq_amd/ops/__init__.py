@@ -1280,3 +1280,95 @@ def softcap(x, cap: float):
     else:
         ref.softcap(x, cap)
     return x
+
+
+# ---------------------------------------------------------------------------
+# Parallel-sublayer residual, rotary windowed differential attention, gated linear
+# recurrences, activated convolutions, softmax top-k routing (csrc/kernels/mix_diff_attn.hip,
+# mix_linrec.hip, mix_par.hip; same library).
+def residual_add_norm(x, y1=None, y2=None, shift=None, w=None, eps: float = 1e-5,
+                      offset: float = 0.0, out=None):
+    """x (fp32, in place) += y1 + y2 + shift (each optional, either dtype; shift is one fp32
+    row added to every row); with ``w``, ``out`` receives rms(x) * (w + offset)."""
+    if _gpu(x):
+        _native.mix_ops().residual_add_norm(x, y1, y2, shift, w, float(eps), float(offset), out)
+    else:
+        ref.residual_add_norm(x, y1, y2, shift, w, eps, offset, out)
+    return out
+
+
+def rotary_inv_freq(rot_dims: int, base: float, device):
+    return ref.rotary_inv_freq(rot_dims, base, device)
+
+
+def rotary_append(qkv, positions, inv_freq, slot_mapping, k_cache, v_cache, H: int, G: int,
+                  maps: int, dim: int, vdim: int, q_out):
+    if _gpu(qkv):
+        _native.mix_ops().rotary_append(qkv, positions, inv_freq, slot_mapping, k_cache, v_cache,
+                                        H, G, maps, dim, vdim, q_out)
+    else:
+        ref.rotary_append(qkv, positions, inv_freq, slot_mapping, k_cache, v_cache, H, G, maps,
+                          dim, vdim, q_out)
+    return q_out
+
+
+DIFF_QBLK = 32       # queries per work item of attn_diff_window (the scheduler's MIXQ_QBLK)
+
+
+def attn_diff_window(q, k_cache, v_cache, block_tables, q_start, q_len, kv_len, work_seq,
+                     work_qblk, gate, out, scale: float, window: int, lam: float, eps: float,
+                     out_mult: float):
+    """Work items (sequence, block of DIFF_QBLK queries) as for attn_mixq_prefill; a decode
+    section's sequences are one work item each (block 0)."""
+    if _gpu(q):
+        _native.mix_ops().attn_diff_window(q, k_cache, v_cache, block_tables, q_start, q_len,
+                                           kv_len, work_seq, work_qblk, gate, out, float(scale),
+                                           int(window), float(lam), float(eps), float(out_mult))
+    else:
+        ref.attn_diff_window(q, k_cache, v_cache, block_tables, q_start, q_len, kv_len, gate, out,
+                             scale, window, lam, eps, out_mult)
+    return out
+
+
+def conv_act_heads(x, w, state, row_state, row_back, row_fwd, positions, n_unit: int, dim: int,
+                   unit_eps: float, out):
+    if _gpu(x):
+        _native.mix_ops().conv_act_heads(x, w, state, row_state, row_back, row_fwd, positions,
+                                         int(n_unit), int(dim), float(unit_eps), out)
+    else:
+        ref.conv_act_heads(x, w, state, row_state, row_back, row_fwd, positions, n_unit, dim,
+                           unit_eps, out)
+    return out
+
+
+def gated_linear_recurrence(q, k, v, z, rate, zbias, zsign: float, beta, gate, gate_sigmoid: bool,
+                            norm_w, eps: float, q_scale: float, state, row_state, row_back,
+                            row_fwd, positions, out, run_rows=None):
+    """``run_rows`` (int32): the first row of every run of the step (-1: none); the kernel
+    launches one workgroup per (run, head)."""
+    if _gpu(q):
+        _native.mix_ops().gated_linear_recurrence(
+            q, k, v, z, rate, zbias, float(zsign), beta, gate, bool(gate_sigmoid), norm_w,
+            float(eps), float(q_scale), state, row_state, row_back, row_fwd, positions, run_rows,
+            out)
+    else:
+        ref.gated_linear_recurrence(q, k, v, z, rate, zbias, zsign, beta, gate, gate_sigmoid,
+                                    norm_w, eps, q_scale, state, row_state, row_back, row_fwd,
+                                    positions, out)
+    return out
+
+
+def moe_route_topk(z, bias, top: int, ids, weights):
+    if _gpu(z):
+        _native.mix_ops().moe_route_topk(z, bias, int(top), ids, weights)
+    else:
+        ref.moe_route_topk(z, bias, top, ids, weights)
+
+
+def gelu_rows(x, out=None):
+    out = torch.empty_like(x) if out is None else out
+    if _gpu(x):
+        _native.mix_ops().gelu_rows(x, out)
+    else:
+        ref.gelu_rows(x, out)
+    return out

@@ -503,3 +503,200 @@ def moe_experts(h, ids, weights, w13, w2, base, out) -> None:
         wt = (weights[rows] * hit[rows]).sum(-1)
         acc[rows] += wt[:, None] * y
     out.copy_(acc)
+
+
+# ---------------------------------------------------------------------------
+# Parallel-sublayer residual, rotary windowed differential attention, gated linear
+# recurrences (plain and delta rule), activated causal convolutions, softmax top-k routing.
+def residual_add_norm(x, y1, y2, shift, w, eps: float, offset: float, out) -> None:
+    """x (fp32, in place) += y1 + y2 + shift (each optional; shift is one row for all);
+    with ``w``: out = x / sqrt(mean(x^2) + eps) * (w + offset) in out's dtype."""
+    for y in (y1, y2, shift):
+        if y is not None:
+            x.add_(y.float())
+    if w is not None:
+        out.copy_((_rms(x, eps) * (w.float() + offset)).to(out.dtype))
+
+
+def rotary_inv_freq(rot_dims: int, base: float, device="cpu") -> torch.Tensor:
+    """f_i = base^(-2i / rot_dims), i < rot_dims / 2, rounded once from float64."""
+    i = torch.arange(rot_dims // 2, dtype=torch.float64)
+    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / max(1, rot_dims)) \
+        .float().to(device)
+
+
+def _rotate_pairs(x, positions, inv_freq):
+    """Rotates the leading 2 * len(inv_freq) entries of the last axis of x [T, ..., w]:
+    entries (2i, 2i+1) by the angle position * f_i (angles, sines and cosines in fp32)."""
+    n = inv_freq.numel()
+    if n == 0:
+        return x
+    ang = positions.float()[:, None] * inv_freq.float()[None]
+    shape = (x.shape[0],) + (1,) * (x.dim() - 2) + (n,)
+    c, s = torch.cos(ang).view(shape), torch.sin(ang).view(shape)
+    x = x.clone()
+    u, v = x[..., 0:2 * n:2].clone(), x[..., 1:2 * n:2].clone()
+    x[..., 0:2 * n:2] = u * c - v * s
+    x[..., 1:2 * n:2] = v * c + u * s
+    return x
+
+
+def rotary_append(qkv, positions, inv_freq, slot_mapping, k_cache, v_cache, H: int, G: int,
+                  maps: int, dim: int, vdim: int, q_out) -> None:
+    """Rows of qkv are q [H, maps, dim] | k [G, maps, dim] | v [G, vdim].  The first
+    2 * len(inv_freq) dimensions of every map of q and k are rotated by the row's position;
+    q goes to q_out [T, H, maps * dim] fp32, k and v into their pages (slot < 0: nowhere)."""
+    T = qkv.shape[0]
+    if T == 0:
+        return
+    nq, nk = H * maps * dim, G * maps * dim
+    x = qkv.float()
+    q = _rotate_pairs(x[:, :nq].reshape(T, H, maps, dim), positions[:T], inv_freq)
+    k = _rotate_pairs(x[:, nq:nq + nk].reshape(T, G, maps, dim), positions[:T], inv_freq)
+    v = x[:, nq + nk:nq + nk + G * vdim].reshape(T, G, vdim)
+    q_out.copy_(q.reshape(T, H, maps * dim))
+    BS = k_cache.shape[2]
+    for t in range(T):
+        s = int(slot_mapping[t])
+        if s >= 0:
+            k_cache[s // BS, :, s % BS] = k[t].reshape(G, maps * dim).to(k_cache.dtype)
+            v_cache[s // BS, :, s % BS] = v[t].to(v_cache.dtype)
+
+
+def attn_diff_window(q, k_cache, v_cache, block_tables, q_start, q_len, kv_len, gate, out,
+                     scale: float, window: int, lam: float, eps: float, out_mult: float) -> None:
+    """Differential attention inside a sliding window.  q [T, H, 2 dim] fp32 (rotated),
+    k_cache [blocks, G, BS, 2 dim], v_cache [blocks, G, BS, vdim]; per head two softmax
+    attentions a1, a2 (the two halves of q and k) over the same values; position i sees
+    j <= i with i - j < window (0: all).  o = a1 - lam a2, divided by its root mean square
+    over vdim (+ eps), times out_mult, times sigmoid(gate[t, h]); out [T, H vdim]."""
+    H, dim = q.shape[1], q.shape[2] // 2
+    G = k_cache.shape[1]
+    rep = H // G
+    for b in range(q_len.shape[0]):
+        ql, kl, t0 = int(q_len[b]), int(kv_len[b]), int(q_start[b])
+        if ql == 0:
+            continue
+        lo = max(0, kl - ql - window + 1) if window > 0 else 0
+        k = _gather_kv(k_cache, block_tables[b], kl).float()[:, lo:].repeat_interleave(rep, 0)
+        v = _gather_kv(v_cache, block_tables[b], kl).float()[:, lo:].repeat_interleave(rep, 0)
+        i = torch.arange(kl - ql, kl)[:, None]
+        j = torch.arange(lo, kl)[None, :]
+        ok = (j <= i) & ((i - j < window) if window > 0 else (j >= 0))
+        qq = q[t0:t0 + ql].float()
+        a = []
+        for mp in range(2):
+            s = torch.einsum("qhe,hke->hqk", qq[:, :, mp * dim:(mp + 1) * dim],
+                             k[:, :, mp * dim:(mp + 1) * dim]) * scale
+            s = s.masked_fill(~ok[None], float("-inf"))
+            a.append(torch.einsum("hqk,hkd->qhd", torch.softmax(s, -1), v))
+        o = _rms(a[0] - lam * a[1], eps) * out_mult
+        o = o * torch.sigmoid(gate[t0:t0 + ql].float())[:, :, None]
+        out[t0:t0 + ql].copy_(o.reshape(ql, -1).to(out.dtype))
+
+
+def conv_act_heads(x, w, state, row_state, row_back, row_fwd, positions, n_unit: int, dim: int,
+                   unit_eps: float, out) -> None:
+    """out[t] = silu(sum_j w[:, j] x[t - (taps-1-j)]) over the sequence of row t (inputs
+    before the run from the state half, zeros before position 0; the run's last taps-1
+    inputs go to the other half; state [2 * slots, taps-1, C] fp32).  The first ``n_unit``
+    heads of ``dim`` channels are then made unit vectors: y / sqrt(sum(y^2) + unit_eps).
+    out [T, C] fp32."""
+    T, C = x.shape
+    if T == 0:
+        return
+    taps = w.shape[1]
+    K = taps - 1
+    S = state.shape[0] // 2
+    xf, wf = x.float(), w.float()
+    acc = torch.zeros(T, C)
+    new = {}
+    for t in range(T):
+        code, i, f, p = int(row_state[t]), int(row_back[t]), int(row_fwd[t]), int(positions[t])
+        rd, wr = _state_rows(code, S) if code >= 0 else (-1, -1)
+        for dl in range(taps):
+            if dl <= i:
+                src = xf[t - dl]
+            elif p - dl >= 0 and rd >= 0:
+                src = state[rd, K + i - dl]
+            else:
+                continue
+            acc[t] += wf[:, taps - 1 - dl] * src
+        if code >= 0:
+            n = i + f + 1
+            if f < K:
+                new[(wr, K - 1 - f)] = xf[t].clone()
+            if i == 0:
+                for e in range(0, K - n):
+                    new[(wr, e)] = state[rd, e + n].clone()
+    for (wr, e), v in new.items():
+        state[wr, e] = v
+    y = torch.nn.functional.silu(acc)
+    if n_unit > 0:
+        u = y[:, :n_unit * dim].reshape(T, n_unit, dim)
+        y[:, :n_unit * dim] = (u / torch.sqrt((u * u).sum(-1, keepdim=True) + unit_eps)).reshape(T, -1)
+    out.copy_(y)
+
+
+def gated_linear_recurrence(q, k, v, z, rate, zbias, zsign: float, beta, gate, gate_sigmoid: bool,
+                            norm_w, eps: float, q_scale: float, state, row_state, row_back,
+                            row_fwd, positions, out) -> None:
+    """Per head a dim x vdim state S (fp32), token by token inside each scheduled run:
+        a_t = exp(-rate_h softplus(zsign (z_t + zbias)))            decay per key channel
+        S <- diag(a_t) S
+        u_t = beta_t (v_t - S^T k_t)   (delta rule; without beta: u_t = v_t)
+        S <- S + k_t u_t^T ;  o_t = q_scale S^T q_t
+    out_t = o_t / rms(o_t) * norm_w * act(gate_t), act = sigmoid or silu.  q, k
+    [T, Hq, dim] (head h reads head h // (H / Hq)), v [T, H, vdim], z [T, H dim], beta
+    [T, H] logits (sigmoid applied here) or None, gate [T, H vdim], norm_w [vdim].
+    state [2 * slots, H, dim, vdim]: read at the run's start (zeros at position 0), the
+    run's last state written to the other half."""
+    T = q.shape[0]
+    if T == 0:
+        return
+    H, dim, vdim = state.shape[1], state.shape[2], state.shape[3]
+    Hq = q.shape[1]
+    rep = H // Hq
+    S_ = state.shape[0] // 2
+    qf = q.float().repeat_interleave(rep, 1)
+    kf = k.float().repeat_interleave(rep, 1)
+    vf = v.float().reshape(T, H, vdim)
+    zz = zsign * (z.float() + zbias.float())
+    a = torch.exp(-rate.float()[None, :, None] * torch.nn.functional.softplus(zz).reshape(T, H, dim))
+    bt = torch.sigmoid(beta.float()) if beta is not None else None
+    o = torch.zeros(T, H, vdim)
+    cur = None
+    for t in range(T):
+        code, i, f, p = int(row_state[t]), int(row_back[t]), int(row_fwd[t]), int(positions[t])
+        if i == 0:
+            cur = state[_state_rows(code, S_)[0]].clone() if p > 0 and code >= 0 \
+                else torch.zeros(H, dim, vdim)
+        cur = a[t][:, :, None] * cur
+        u = vf[t]
+        if bt is not None:
+            u = bt[t][:, None] * (u - torch.einsum("hkv,hk->hv", cur, kf[t]))
+        cur = cur + kf[t][:, :, None] * u[:, None, :]
+        o[t] = torch.einsum("hkv,hk->hv", cur, qf[t]) * q_scale
+        if f == 0 and code >= 0:
+            state[_state_rows(code, S_)[1]] = cur
+    g = gate.float().reshape(T, H, vdim)
+    g = torch.sigmoid(g) if gate_sigmoid else torch.nn.functional.silu(g)
+    y = _rms(o, eps) * norm_w.float() * g
+    out.copy_(y.reshape(T, H * vdim).to(out.dtype))
+
+
+def moe_route_topk(z, bias, top: int, ids, weights) -> None:
+    """The ``top`` largest of z + bias per row (ties to the lower index), weighted by the
+    softmax over the chosen logits only."""
+    zz = z.float() + (bias.float() if bias is not None else 0.0)
+    T, E = zz.shape
+    order = torch.argsort(zz, dim=-1, descending=True, stable=True)[:, :top]
+    val = torch.gather(zz, 1, order)
+    ids.copy_(order.to(ids.dtype))
+    weights.copy_(torch.softmax(val, -1))
+
+
+def gelu_rows(x, out) -> None:
+    """out = 0.5 x (1 + erf(x / sqrt 2)), computed in fp32."""
+    xf = x.float()
+    out.copy_((0.5 * xf * (1.0 + torch.erf(xf * 0.7071067811865476))).to(out.dtype))
