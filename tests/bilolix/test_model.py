@@ -1,0 +1,301 @@
+"""Whole Bilolix models through the engine (scheduler, paged cache, state slots) against the
+slow oracle: whole prompts, token-by-token decoding, portions, mixed batches with pages and
+slots reused, window edges in prompts and in decoding, greedy generation."""
+import pytest
+import torch
+
+from . import oracle
+from .common import (NO_LOOP, ONE_PASS, REGS, SMALL, alone, attention, build, check, config, delta,
+                     dense, gla, moe, run_schedule, tokens)
+
+DEVICES = ["cpu", pytest.param("cuda:0", marks=pytest.mark.gpu)]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("cfg", [SMALL, REGS, NO_LOOP, ONE_PASS], ids=["small", "regs", "noloop", "onepass"])
+def test_whole_prompt_and_token_by_token(device, cfg):
+    eng, full = build(cfg, device)
+    if device != "cpu":
+        assert eng.model.w["embed"].is_cuda
+    t = tokens(75, cfg["vocab"], 1)
+    check(run_schedule(eng, alone(t, [])), cfg, full, {"a": t})
+    check(run_schedule(eng, alone(t, [40] + [1] * 35)), cfg, full, {"a": t})
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_residual_stream_after_every_layer_run(device):
+    """A looped layer counts once per pass; the step vector of a pass belongs to the pass's
+    first layer, not to the layer before it."""
+    cfg = SMALL
+    eng, full = build(cfg, device)
+    t = tokens(45, cfg["vocab"], 3)
+    want = []
+    oracle.forward(cfg, full, t, want)
+    taps, fwd = [], eng.model.forward
+    eng.model.forward = lambda m: fwd(m, taps)
+    try:
+        run_schedule(eng, alone(t, []))
+    finally:
+        eng.model.forward = fwd
+    assert len(taps) == len(want) == 1 + 3 * 3 + 2
+    for i, (a, b) in enumerate(zip(taps, want)):
+        err = float((a.double().cpu() - b).abs().max() / b.abs().max())
+        assert err < 1e-4, f"layer run {i}: {err:.2e}"
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("cuts", [[2] * 30, [3, 2, 33, 2, 5, 31, 2], [32, 32, 1, 1, 2], [64, 2],
+                                  [7, 7, 7, 7, 7, 7, 7, 7, 7, 7, 2, 1, 1]])
+def test_portions(device, cuts):
+    """Portions down to two tokens, cut inside pages, windows and the convolutions' reach;
+    short ones run in the decode section (<= 32 rows), long ones in the prefill section."""
+    eng, full = build(SMALL, device)
+    t = tokens(90, SMALL["vocab"], 2)
+    check(run_schedule(eng, alone(t, cuts)), SMALL, full, {"a": t})
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_first_tokens_and_one_token_requests(device):
+    eng, full = build(REGS, device)
+    for n in (1, 2, 3, 5):
+        t = tokens(n, REGS["vocab"], 10 + n)
+        check(run_schedule(eng, alone(t, [])), REGS, full, {"a": t})
+        check(run_schedule(eng, alone(t, [1] * n)), REGS, full, {"a": t})
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_batches_of_unequal_requests(device):
+    """Up to four live requests, portions beside single tokens, requests that pause, pages and
+    slots given back and used again by later requests: each row as if its request ran alone."""
+    cfg = SMALL
+    eng, full = build(cfg, device, max_kv_blocks=14)       # 13 pages: reuse is forced
+    V = cfg["vocab"]
+    req = {n: tokens(L, V, 20 + i) for i, (n, L) in enumerate(
+        [("a", 97), ("b", 40), ("c", 5), ("d", 66), ("e", 130), ("f", 33), ("g", 64)])}
+    at = {n: 0 for n in req}
+
+    def take(n, c):
+        lo = at[n]
+        at[n] = lo + c
+        return (n, req[n][lo:lo + c], list(range(c)))
+
+    plan = [
+        [("a", 50), ("b", 2), ("c", 5)], [("a", 1), ("b", 33), ("d", 40)], [("a", 1), ("b", 5)],
+        [("a", 45), ("d", 2)], [("d", 24), ("e", 64), ("f", 3)], [("e", 1), ("f", 30)],
+        [("e", 2), ("g", 64)], [("e", 63)],
+    ]
+    steps = []
+    for st in plan:
+        entries = [take(n, c) for n, c in st]
+        steps.append({"entries": entries, "end": [n for n, _ in st if at[n] == len(req[n])]})
+    assert all(at[n] == len(req[n]) for n in req)
+    got = run_schedule(eng, steps)
+    check(got, cfg, full, req)
+    assert len(got) == sum(len(t) for t in req.values())
+    assert eng.core.num_free_state_slots == 4 and eng.core.num_free_blocks == 13
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_slot_and_pages_reused_after_release(device):
+    """One slot, pool of one request: each request runs where the last one's state matrices,
+    convolution inputs and keys still lie."""
+    cfg = REGS
+    eng, full = build(cfg, device, max_num_seqs=1, max_kv_blocks=4)
+    for i in range(3):
+        t = tokens(70 + i, cfg["vocab"], 40 + i)
+        check(run_schedule(eng, alone(t, [33, 2, 1, 1])), cfg, full, {"a": t})
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_long_decoding_over_page_and_window_edges(device):
+    cfg = SMALL
+    eng, full = build(cfg, device)
+    t = tokens(140, cfg["vocab"], 50)
+    check(run_schedule(eng, alone(t, [20] + [1] * 120)), cfg, full, {"a": t})
+
+
+def _sharp(cfg, window_layer=0, boost=6.0):
+    """Weights whose attention layer has sharp scores (queries and keys scaled up), so that a
+    key that enters or leaves the window moves the logits visibly."""
+    _, full = build(cfg, "cpu")
+    full = dict(full)
+    p = f"l{window_layer}.mix."
+    full[p + "q"] = (full[p + "q"] * boost).bfloat16().float()
+    full[p + "k"] = (full[p + "k"] * boost).bfloat16().float()
+    return full
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("window", [1, 2, 31, 32, 33, 64, 70])
+def test_window_edges_with_sharp_scores(device, window):
+    """Windows of one key, at, just under and just over the page size and a multiple of it:
+    with sharp scores one key more or less in view shows; prompt rows and decoded rows."""
+    cfg = config([attention(2, 1, 16, 16, window, 8, None, scale=0.5),
+                  attention(4, 4, 8, 8, window + 1, 8, dense(16), scale=0.5)], width=32, vocab=50)
+    full = _sharp(cfg)
+    eng, _ = build(cfg, device, full=full)
+    t = tokens(150, cfg["vocab"], 60 + window)
+    got = run_schedule(eng, alone(t, [75, 2, 31] + [1] * 42))
+    check(got, cfg, full, {"a": t})
+    # the mask matters: a window one key wider gives visibly other logits
+    wider = config([attention(2, 1, 16, 16, window + 1, 8, None, scale=0.5),
+                    attention(4, 4, 8, 8, window + 1, 8, dense(16), scale=0.5)], width=32, vocab=50)
+    other = oracle.forward(wider, full, t)
+    mine = torch.stack([got[("a", p)].double() for p in range(150)])
+    assert float((other - mine).abs().max()) > 1e-2
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_far_key_without_window(device):
+    """window 0 = every earlier key: sharp scores over hundreds of keys across many pages, in a
+    prompt and in decoding."""
+    cfg = config([attention(3, 1, 16, 8, 0, 16, dense(16), scale=0.4), gla(2, 8, 8, 4.0, None)],
+                 width=32, vocab=50)
+    full = _sharp(cfg, boost=4.0)
+    eng, _ = build(cfg, device, full=full, max_kv_blocks=40, max_model_len=1024, max_batched_tokens=1024)
+    t = tokens(400, cfg["vocab"], 77)
+    check(run_schedule(eng, alone(t, [330, 2, 31] + [1] * 37)), cfg, full, {"a": t})
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_state_carries_a_far_token(device):
+    """Slow decays: a token hundreds of positions back still shows in the recurrent layers'
+    outputs, through portions and decoding."""
+    cfg = config([gla(2, 16, 16, 64.0, None), delta(2, 1, 16, 16, 3, None)], width=32, vocab=50)
+    _, full = build(cfg, "cpu")
+    full = dict(full)
+    full["l0.mix.a2.b"] = full["l0.mix.a2.b"] + 4.0            # sigmoid ~ 1: almost no decay
+    full["l1.mix.A_log"] = full["l1.mix.A_log"] - 4.0          # tiny rate
+    eng, _ = build(cfg, device, full=full, max_kv_blocks=40, max_model_len=1024, max_batched_tokens=1024)
+    t = tokens(300, cfg["vocab"], 78)
+    got = run_schedule(eng, alone(t, [250, 2, 17] + [1] * 31))
+    check(got, cfg, full, {"a": t})
+    t2 = list(t)
+    t2[3] = (t2[3] + 1) % cfg["vocab"]
+    other = oracle.forward(cfg, full, t2)
+    assert float((other[-1] - got[("a", 299)].double()).abs().max()) > 1e-3
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_bfloat16_close_to_oracle_and_independent_of_cuts(device):
+    cfg = SMALL
+    eng, full = build(cfg, device, dtype=torch.bfloat16)
+    a, b = tokens(100, cfg["vocab"], 80), tokens(41, cfg["vocab"], 81)
+    steps = [{"entries": [("a", a[:70], list(range(70))), ("b", b[:3], [0, 1, 2])], "end": []},
+             {"entries": [("a", a[70:71], [0]), ("b", b[3:40], list(range(37)))], "end": []},
+             {"entries": [("a", a[71:], list(range(29))), ("b", b[40:], [0])], "end": ["a", "b"]}]
+    got = run_schedule(eng, steps)
+    assert len(got) == 141
+    ref = {"a": oracle.forward(cfg, full, a), "b": oracle.forward(cfg, full, b)}
+
+    def err(row, want, std):
+        d = row.double() - want.double()
+        d = d - d.mean()
+        return float(d.pow(2).mean().sqrt() / std)
+
+    # a rounded router input can flip a close choice of experts at a single position: nearly
+    # all rows are within rounding of the oracle, and the typical row is far inside
+    e = sorted(err(row, ref[n][p], ref[n].std()) for (n, p), row in got.items())
+    assert e[len(e) // 2] < 0.04 and e[int(len(e) * 0.95)] < 0.12, (e[len(e) // 2], e[-8:])
+    whole = run_schedule(eng, alone(a, []))
+    e = sorted(err(whole[("a", p)], got[("a", p)], ref["a"].std()) for p in range(100))
+    assert e[50] < 0.04 and e[95] < 0.12, (e[50], e[-8:])
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_greedy_generation_through_the_engine(device):
+    """generate() (scheduler, sampler at temperature 0, decode steps) picks the oracle's tokens."""
+    from replisense_rfq_amd.engine.sequence import SamplingParams
+
+    cfg = REGS
+    eng, full = build(cfg, device)
+    prompts = [tokens(n, cfg["vocab"], 70 + n) for n in (9, 35, 2)]
+    seqs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, grammar=False))
+    for p, s in zip(prompts, seqs):
+        assert s.output_ids == oracle.greedy(cfg, full, p, 10)
+    assert eng.core.num_free_state_slots == 4
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_checkpoint_folder_round_trip(device, tmp_path):
+    """config.json + model.safetensors written to a folder choose the model class and load."""
+    import json
+
+    from safetensors.torch import save_file
+
+    from replisense_rfq_amd.engine.engine import LLMEngine
+    from replisense_rfq_amd.utils.config import EngineConfig
+
+    cfg = NO_LOOP if device == "cpu" else SMALL
+    _, full = build(cfg, "cpu")
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in full.items()},
+              str(tmp_path / "model.safetensors"))
+    eng = LLMEngine(EngineConfig(model="x", weights_path=str(tmp_path), dtype="float32", device=str(device),
+                                 max_num_seqs=2, max_kv_blocks=8, max_batched_tokens=128,
+                                 max_model_len=128, use_graphs=False, grammar=False,
+                                 prefix_cache=False, warm_prefix=False, tune_gemm=False,
+                                 jump_forward=False))
+    assert type(eng.model).__name__ == "BilolixLM"
+    t = tokens(20, cfg["vocab"], 5)
+    check(run_schedule(eng, alone(t, [9, 2])), cfg, full, {"a": t})
+
+
+def test_named_configuration_and_registry():
+    from replisense_rfq_amd.models import layered_model_class
+    from replisense_rfq_amd.models.config import get_config
+
+    c = get_config("tiny-bilolix")
+    assert c.architecture == "Bilolix" and len(c.runs) == len(c.layers) + 2
+    assert layered_model_class("Bilolix").__name__ == "BilolixLM"
+    assert c.params() > 0 and c.kv_bytes_per_token() > 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_decode_graphs_replayed_between_eager_steps(dtype):
+    """Decode steps replay a captured hipGraph (rotation, windowed attention, convolutions,
+    recurrences, routing and experts inside it), prompts run eagerly in between: greedy
+    generation of several waves of requests picks the oracle's tokens each time (fp32), and
+    the graph was the path that ran."""
+    from replisense_rfq_amd.engine.sequence import SamplingParams
+
+    cfg = REGS
+    eng, full = build(cfg, "cuda:0", dtype=dtype, use_graphs=True, graph_buckets=(4,))
+    assert eng.runner.graphs
+    for wave in range(3):
+        prompts = [tokens(n, cfg["vocab"], 100 + 10 * wave + n) for n in (9, 35, 2)]
+        seqs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, grammar=False))
+        if dtype == torch.float32:
+            for p, s in zip(prompts, seqs):
+                assert s.output_ids == oracle.greedy(cfg, full, p, 10), wave
+    assert eng.runner.stats["graph_steps"] >= 24
+    assert eng.core.num_free_state_slots == 4
+
+
+@pytest.mark.gpu
+def test_layer_sized_model_in_bf16_against_the_torch_ops():
+    """Layers of a served model's widths (128-wide maps, 64- and 128-wide recurrent heads,
+    experts on the grouped GEMMs), bf16 on the GPU: prompts in portions and decoding, against
+    the same weights run in fp32 through the torch ops on the CPU."""
+    cfg = config([attention(8, 2, 128, 128, 200, 64, moe(512, 8, 2), scale=128 ** -0.5),
+                  gla(8, 64, 128, 16.0, dense(2048)),
+                  delta(8, 4, 128, 128, 4, moe(512, 8, 2))], vocab=1000, width=1024, loop=(0, 2, 2))
+    kw = dict(max_kv_blocks=40, max_model_len=640, max_batched_tokens=1024, ranks=(32, 64))
+    ref_eng, full = build(cfg, "cpu", **kw)
+    eng, _ = build(cfg, "cuda:0", dtype=torch.bfloat16, full=full, **kw)
+    a, b = tokens(420, cfg["vocab"], 90), tokens(130, cfg["vocab"], 91)
+    steps = [{"entries": [("a", a[:300], [299]), ("b", b[:100], [0, 99])], "end": []},
+             {"entries": [("a", a[300:400], [0, 99]), ("b", b[100:101], [0])], "end": []}]
+    steps += [{"entries": [("a", a[400 + i:401 + i], [0]), ("b", b[101 + i:102 + i], [0])], "end": []}
+              for i in range(20)]
+    want = run_schedule(ref_eng, steps)
+    got = run_schedule(eng, steps)
+    assert len(got) == len(want) == 46
+    e = []
+    for key, row in got.items():
+        d = row.double() - want[key].double()
+        d = d - d.mean()
+        e.append(float(d.pow(2).mean().sqrt() / want[key].double().std()))
+    e.sort()
+    assert e[len(e) // 2] < 0.05 and e[-3] < 0.15, e[-6:]
