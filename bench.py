@@ -366,8 +366,8 @@ def main():
     args = parse()
     t_start = time.perf_counter()
     if args.arch_compare:
-        if args.arch_compare not in ("livisun", "numalorn") or args.gpus != 1:
-            raise SystemExit("bench: --arch-compare livisun | numalorn runs on one GPU")
+        if args.arch_compare not in ("livisun", "numalorn", "bilolix") or args.gpus != 1:
+            raise SystemExit("bench: --arch-compare livisun | numalorn | bilolix runs on one GPU")
         from replisense_rfq_amd.benchmarks import arch_compare
 
         extra = {}
@@ -376,6 +376,10 @@ def main():
             from replisense_rfq_amd.benchmarks import arch_kernels
 
             extra["kernels"] = arch_kernels.run(args)
+        if args.arch_compare == "bilolix" and not args.arch_models:
+            from replisense_rfq_amd.benchmarks import arch_kernels
+
+            extra["kernels"] = arch_kernels.run_bilolix(args)
         print(json.dumps({"metric": "arch_compare", "arch": args.arch_compare, "dtype": "bf16",
                           "data": "synthetic", **arch_compare.run(args), **extra}), flush=True)
         return

@@ -1,7 +1,9 @@
 """Prefill and decode throughput of a layer-list model beside the closest decoder of the
-framework at equal layer sizes: ``bench.py --arch-compare livisun`` (beside Llama) and
+framework at equal layer sizes: ``bench.py --arch-compare livisun`` (beside Llama),
 ``--arch-compare numalorn`` (beside the Mixtral-style sparse decoder: same width, head count,
-experts, choices per token and expert width).
+experts, choices per token and expert width) and ``--arch-compare bilolix`` (beside Numalorn:
+same width, head count, experts and expert width; attention and recurrent layers alternate
+in both).
 
 Both run through the same engine (scheduler, paged cache, hipGraph decode steps), with
 random weights, a few layers of a real model's shape and a small vocabulary, so the numbers
@@ -57,6 +59,26 @@ def _moe_configs(name, d, H, G, E, top, F):
     return sparse, num
 
 
+def _bilolix_configs(name, d, H, G, E, top, F):
+    """Numalorn and Bilolix at equal sizes.  Bilolix: differential attention with two 64-wide
+    score maps per head (128-wide queries and keys, as wide as Numalorn's heads), 128-wide
+    values, a window of 1,024 positions, alternating with a gla layer and a channel_delta
+    layer of d/128 heads with 64 x 128 states; the same experts in every layer."""
+    from ..models.config import bilolix_layers, numalorn_layers
+
+    num = LayeredConfig(f"cmp-numalorn-{name}", architecture="Numalorn", vocab_size=VOCAB,
+                        hidden=d, canon_taps=0, residual_mult=0.5, logit_softcap=30.0,
+                        decay_rank=64,
+                        layers=numalorn_layers(LAYERS, H, 128, 128, 3 * d // 8, 512, d // 64, F, E,
+                                               top, 2, 1, 0))
+    bil = LayeredConfig(f"cmp-bilolix-{name}", architecture="Bilolix", vocab_size=VOCAB, hidden=d,
+                        canon_taps=0, decay_rank=64, gate_rank=64, loop=(0, 0, 1),
+                        layers=bilolix_layers("agac"[:LAYERS], H, G, 64, 128, 0, experts=E, top=top,
+                                              expert_ff=F, window=1024, rot_dims=64, rot_base=5e5,
+                                              rec_heads=d // 128, rec_dim=64, moe_every=1))
+    return num, bil
+
+
 def _engine(mcfg, args, batch):
     from ..models import layered_model_class
     from ..models.llama import DecoderLM
@@ -66,6 +88,11 @@ def _engine(mcfg, args, batch):
         from ..models.weights import init_numalorn_weights
 
         w = init_numalorn_weights(mcfg, dev, torch.bfloat16, args.seed, keep_full=False)
+        model = layered_model_class(mcfg.architecture)(mcfg, dev, weights=w)
+    elif isinstance(mcfg, LayeredConfig) and mcfg.architecture == "Bilolix":
+        from ..models.weights import init_bilolix_weights
+
+        w = init_bilolix_weights(mcfg, dev, torch.bfloat16, args.seed, keep_full=False)
         model = layered_model_class(mcfg.architecture)(mcfg, dev, weights=w)
     elif isinstance(mcfg, LayeredConfig):
         model = layered_model_class(mcfg.architecture)(mcfg, dev, seed=args.seed)
@@ -107,15 +134,16 @@ def run(args) -> dict:
            "decode": [64, 128], "sizes": {}}
     only = [x for x in getattr(args, "arch_sizes", "").split(",") if x]
     arch = getattr(args, "arch_compare", "livisun")
-    base = "llama" if arch == "livisun" else "sparse"
+    base = {"livisun": "llama", "numalorn": "sparse", "bilolix": "numalorn"}[arch]
+    make = {"livisun": _configs, "numalorn": _moe_configs, "bilolix": _bilolix_configs}[arch]
     for size in (SIZES if arch == "livisun" else MOE_SIZES):
         name = size[0]
         if only and name not in only:
             continue
         row = {}
         models = [x for x in getattr(args, "arch_models", "").split(",") if x]
-        for mcfg in (_configs(*size) if arch == "livisun" else _moe_configs(*size)):
-            kind = arch if isinstance(mcfg, LayeredConfig) else base
+        for mcfg in make(*size):
+            kind = mcfg.architecture.lower() if isinstance(mcfg, LayeredConfig) else base
             if models and kind not in models:
                 continue
             print(f"[arch-compare] {name}: {kind}", file=sys.stderr, flush=True)

@@ -164,3 +164,129 @@ def run(args) -> dict:
     _experts(64, d, F, E, top, dec)
     res["decode_step_64_rows"] = dec
     return res
+
+
+# ---------------------------------------------------------------------------
+# Bilolix's layer kernels at the same step sizes (``bench.py --arch-compare bilolix``):
+# 4096-wide layers, 32 heads with two 64-wide score maps over 8 key/value heads and 128-wide
+# values, a window of 1,024 positions, 32 recurrent heads with 64 x 128 states, a convolution
+# of 4 taps; beside them Numalorn's like kernels (the entries of ``run`` above).
+def _b_rows(T, d, out):
+    g = torch.Generator(device=DEV).manual_seed(0)
+    x = torch.randn(T, d, generator=g, device=DEV)
+    y1 = torch.randn(T, d, generator=g, device=DEV).bfloat16()
+    y2 = torch.randn(T, d, generator=g, device=DEV)
+    w = torch.randn(d, generator=g, device=DEV) * 0.3
+    h = torch.empty(T, d, dtype=torch.bfloat16, device=DEV)
+    out["residual_add_norm"] = _entry(_time(lambda: ops.residual_add_norm(x, y1, y2, None, w, 1e-5, 1.0, h)),
+                                      T * d * 16, 0)
+    F = 14336
+    u = torch.randn(T, F, generator=g, device=DEV).bfloat16()
+    o = torch.empty_like(u)
+    out["gelu_rows"] = _entry(_time(lambda: ops.gelu_rows(u, o)), T * F * 4, 0)
+    z = torch.randn(T, 8, generator=g, device=DEV) * 2
+    b = torch.randn(8, generator=g, device=DEV)
+    ids = torch.empty(T, 2, dtype=torch.int32, device=DEV)
+    wts = torch.empty(T, 2, device=DEV)
+    out["moe_route_topk"] = _entry(_time(lambda: ops.moe_route_topk(z, b, 2, ids, wts)), T * (8 * 4 + 16), 0)
+
+
+def _b_attention(H, G, dim, vdim, window, lens, q_lens, out, name):
+    g = torch.Generator(device=DEV).manual_seed(2)
+    BS = 32
+    nblk = sum((n + BS - 1) // BS for n in lens) + 1
+    kc = (torch.randn(nblk, G, BS, 2 * dim, generator=g, device=DEV) * 0.5).bfloat16()
+    vc = (torch.randn(nblk, G, BS, vdim, generator=g, device=DEV) * 0.5).bfloat16()
+    T = sum(q_lens)
+    N = (H + G) * 2 * dim + G * vdim
+    qkv = (torch.randn(T, N, generator=g, device=DEV) * 0.5).bfloat16()
+    pos = torch.cat([torch.arange(n - q, n) for n, q in zip(lens, q_lens)]).to(torch.int32).to(DEV)
+    maxb = (max(lens) + BS - 1) // BS
+    tables, at, slots = [], 0, []
+    for n, q in zip(lens, q_lens):
+        nb = (n + BS - 1) // BS
+        tables.append(list(range(at, at + nb)) + [nblk - 1] * (maxb - nb))
+        slots += [(at + p // BS) * BS + p % BS for p in range(n - q, n)]
+        at += nb
+    inv = ops.rotary_inv_freq(dim, 5e5, DEV)
+    q = torch.empty(T, H, 2 * dim, device=DEV)
+    sl = _i32(slots)
+    t = _time(lambda: ops.rotary_append(qkv, pos, inv, sl, kc, vc, H, G, 2, dim, vdim, q))
+    out[f"rotary_append ({name})"] = _entry(t, T * N * 2 + T * H * 2 * dim * 4 + T * G * (2 * dim + vdim) * 2, 0)
+    gate = torch.randn(T, H, generator=g, device=DEV).bfloat16()
+    o = torch.empty(T, H * vdim, dtype=torch.bfloat16, device=DEV)
+    starts = [sum(q_lens[:i]) for i in range(len(lens))]
+    bt, qs, ql, kl = _i32(tables), _i32(starts), _i32(q_lens), _i32(lens)
+    work = [(s, b) for s, n in enumerate(q_lens) for b in range((n + 31) // 32)]
+    ws, wq = _i32([w[0] for w in work]), _i32([w[1] for w in work])
+    pairs = 0
+    for n, ql_ in zip(lens, q_lens):
+        for p in range(n - ql_, n):
+            pairs += min(p + 1, window)
+    flops = (4.0 * dim + 4.0 * vdim) * H * pairs
+    seen = sum(min(n, window + q - 1) for n, q in zip(lens, q_lens))
+    nbytes = seen * G * (2 * dim + vdim) * 2 + T * H * (2 * dim * 4 + vdim * 2)
+    t = _time(lambda: ops.attn_diff_window(q, kc, vc, bt, qs, ql, kl, ws, wq, gate, o, dim ** -0.5,
+                                           window, 0.4, 1e-5, 0.4), reps=5, warm=2)
+    out[f"attn_diff_window ({name})"] = _entry(t, nbytes, flops)
+
+
+def _b_recurrence(T, H, dim, vdim, rows, out, decode):
+    g = torch.Generator(device=DEV).manual_seed(1)
+    run = torch.nonzero(rows[1] == 0)[:, 0].to(torch.int32)
+    seqs = int(run.numel())
+    q, k = ((torch.randn(T, H, dim, generator=g, device=DEV) * 0.5).bfloat16() for _ in range(2))
+    v = (torch.randn(T, H, vdim, generator=g, device=DEV) * 0.5).bfloat16()
+    gate = torch.randn(T, H * vdim, generator=g, device=DEV).bfloat16()
+    z = torch.randn(T, H * dim, generator=g, device=DEV)
+    rate = torch.full((H,), 1 / 16, device=DEV)
+    zb = torch.randn(H * dim, generator=g, device=DEV) + 2
+    nw = torch.ones(vdim, device=DEV)
+    st = torch.zeros(128, H, dim, vdim, device=DEV)
+    y = torch.empty(T, H * vdim, dtype=torch.bfloat16, device=DEV)
+    state_bytes = (2 if decode else 1) * seqs * H * dim * vdim * 4
+    t = _time(lambda: ops.gated_linear_recurrence(q, k, v, z, rate, zb, -1.0, None, gate, False, nw, 1e-5,
+                                                  dim ** -0.5, st, *rows, y, run), reps=5, warm=2)
+    out["gated_linear_recurrence (gla)"] = _entry(
+        t, T * H * (2 * dim * 2 + dim * 4 + vdim * 6) + state_bytes, 6.0 * T * H * dim * vdim)
+    # the delta rule: q, k, v come from the convolution in fp32
+    C = 2 * H * dim + H * vdim
+    x = (torch.randn(T, C, generator=g, device=DEV) * 0.5).bfloat16()
+    cw = torch.randn(C, 4, generator=g, device=DEV) * 0.5
+    cs = torch.zeros(128, 3, C, device=DEV)
+    qkv = torch.empty(T, C, device=DEV)
+    t = _time(lambda: ops.conv_act_heads(x, cw, cs, *rows, 2 * H, dim, 1e-6, qkv))
+    out["conv_act_heads"] = _entry(t, T * C * 6 + (seqs * 3 * C * 8 if decode else 0), 0)
+    beta = torch.randn(T, H, generator=g, device=DEV).bfloat16()
+    qf, kf = qkv[:, :H * dim].unflatten(1, (H, dim)), qkv[:, H * dim:2 * H * dim].unflatten(1, (H, dim))
+    vf = qkv[:, 2 * H * dim:].unflatten(1, (H, vdim))
+    t = _time(lambda: ops.gated_linear_recurrence(qf, kf, vf, z, rate, zb, 1.0, beta, gate, True, nw, 1e-5,
+                                                  dim ** -0.5, st, *rows, y, run), reps=5, warm=2)
+    out["gated_linear_recurrence (delta rule)"] = _entry(
+        t, T * H * (2 * dim * 4 + dim * 4 + vdim * 8) + state_bytes, 10.0 * T * H * dim * vdim)
+
+
+def run_bilolix(args) -> dict:
+    torch.manual_seed(0)
+    d, H, G, dim, vdim, window, RH = 4096, 32, 8, 64, 128, 1024, 32
+    res = {"width": d, "heads": [H, G], "maps": [2, dim], "vdim": vdim, "window": window,
+           "recurrent_heads": [RH, dim, vdim]}
+    pre, like_pre = {}, {}
+    _b_rows(4096, d, pre)
+    rows = _runs([2048, 2048], [0, 63])
+    _b_recurrence(4096, RH, dim, vdim, rows, pre, False)
+    _b_attention(H, G, dim, vdim, window, [2048, 600], [2048, 600], pre, "prefill")
+    nrows = _rows(4096, d, [2048, 2048], [0, 63], like_pre)
+    _wkv(4096, 64, 64, nrows, like_pre, False)
+    _attention(32, 512, [2048, 600], [2048, 600], like_pre, "prefill", mfma=True)
+    res["prefill_step_4096_rows"] = {"bilolix": pre, "numalorn": like_pre}
+    dec, like_dec = {}, {}
+    _b_rows(64, d, dec)
+    rows = _runs([1] * 64, list(range(64)), first=600)
+    _b_recurrence(64, RH, dim, vdim, rows, dec, True)
+    _b_attention(H, G, dim, vdim, window, [600] * 64, [1] * 64, dec, "decode")
+    nrows = _rows(64, d, [1] * 64, list(range(64)), like_dec, first=600)
+    _wkv(64, 64, 64, nrows, like_dec, True)
+    _attention(32, 512, [600] * 64, [1] * 64, like_dec, "decode", mfma=True)
+    res["decode_step_64_rows"] = {"bilolix": dec, "numalorn": like_dec}
+    return res

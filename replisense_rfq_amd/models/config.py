@@ -387,21 +387,22 @@ def bilolix_from_json(d: dict, name: str | None = None) -> LayeredConfig:
 
 def bilolix_layers(order, heads, kv_heads, dim, vdim, ff, experts=0, top=0, expert_ff=0,
                    window=0, rot_dims=None, rot_base=10000.0, diff=0.5, tau=16.0, conv=4,
-                   rec_heads=None, rec_kv_heads=None):
+                   rec_heads=None, rec_kv_heads=None, rec_dim=None, moe_every=2):
     """Layers of the kinds named in ``order`` ("a" differential attention, "g" gla, "c"
-    channel_delta); with experts, every second layer's feed-forward is a mixture."""
+    channel_delta); with experts, every ``moe_every``-th layer's feed-forward is a mixture."""
     rh = rec_heads or heads
     rk = rec_kv_heads or rh
+    rd = rec_dim or dim
     out = []
     for i, c in enumerate(order):
         if c == "a":
             m = MixerSpec("diff_attention", heads, kv_heads, dim, vdim, dim ** -0.5, window=window,
                           rot_dims=dim if rot_dims is None else rot_dims, rot_base=rot_base, diff=diff)
         elif c == "g":
-            m = MixerSpec("gla", rh, rh, dim, vdim, dim ** -0.5, tau=tau)
+            m = MixerSpec("gla", rh, rh, rd, vdim, rd ** -0.5, tau=tau)
         else:
-            m = MixerSpec("channel_delta", rh, rk, dim, vdim, dim ** -0.5, conv=conv)
-        if experts and i % 2 == 1:
+            m = MixerSpec("channel_delta", rh, rk, rd, vdim, rd ** -0.5, conv=conv)
+        if experts and i % moe_every == moe_every - 1:
             f = MlpSpec("moe", expert_ff, 0.0, experts, top, router="softmax_top")
         else:
             f = MlpSpec("gelu", ff, 0.0) if ff else None
