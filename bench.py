@@ -76,7 +76,8 @@ def parse():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--arch-sizes", default="", help="--arch-compare: size classes, comma separated")
     ap.add_argument("--arch-models", default="",
-                    help="--arch-compare: which of the two models to run (default both), comma separated")
+                    help="--arch-compare: which of the two models to run (default both), comma separated; "
+                         "'kernels' (bilolix): only the per-kernel times")
     ap.add_argument("--arch-compare", default="",
                     help="livisun | numalorn: instead of the RFQ workload, time prefill and decode "
                          "of the layer-list model beside the closest decoder at equal layer sizes "
@@ -376,7 +377,7 @@ def main():
             from replisense_rfq_amd.benchmarks import arch_kernels
 
             extra["kernels"] = arch_kernels.run(args)
-        if args.arch_compare == "bilolix" and not args.arch_models:
+        if args.arch_compare == "bilolix" and (not args.arch_models or "kernels" in args.arch_models):
             from replisense_rfq_amd.benchmarks import arch_kernels
 
             extra["kernels"] = arch_kernels.run_bilolix(args)

@@ -77,6 +77,15 @@ void launch_conv_act_heads(bool, const void*, int64_t, const float*, float*, con
 void launch_moe_route_topk(const float*, const float*, int, int, int, int32_t*, float*, hipStream_t);
 void launch_gelu_rows(bool, const void*, int64_t, void*, int64_t, int, int, hipStream_t);
 size_t attn_diff_lds(int);
+bool diff_mfma_ok(int, int, int);
+bool launch_attn_diff_mfma(const float*, const void*, const void*, const int32_t*, int,
+                           const int32_t*, const int32_t*, const int32_t*, const int32_t*,
+                           const int32_t*, int, const void*, int64_t, void*, int64_t, float, int,
+                           float, float, float, int, int, int, int, int, hipStream_t);
+int launch_attn_diff_decode(bool, const float*, const void*, const void*, const int32_t*, int,
+                            const int32_t*, const int32_t*, const int32_t*, int, int, const void*,
+                            int64_t, void*, int64_t, float, int, float, float, float, int, int, int,
+                            int, int, hipStream_t);
 bool launch_attn_diff_window(bool, const float*, const void*, const void*, const int32_t*, int,
                              const int32_t*, const int32_t*, const int32_t*, const int32_t*,
                              const int32_t*, int, const void*, int64_t, void*, int64_t, float, int,
@@ -556,7 +565,7 @@ void attn_diff_window(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
                       const Tensor& bt, const Tensor& q_start, const Tensor& q_len,
                       const Tensor& kv_len, const Tensor& work_seq, const Tensor& work_qblk,
                       const Tensor& gate, const Tensor& out, double scale, int64_t window,
-                      double lam, double eps, double out_mult) {
+                      double lam, double eps, double out_mult, int64_t short_rows, bool mfma) {
   const bool f32 = act_f32(k_cache, "attn_diff_window k_cache");
   TORCH_CHECK(q.dim() == 3 && q.size(2) % 2 == 0, "attn_diff_window: q [T, H, 2 dim]");
   const int T = (int)q.size(0), H = (int)q.size(1), dim = (int)q.size(2) / 2;
@@ -576,6 +585,32 @@ void attn_diff_window(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
   TORCH_CHECK(out.is_cuda() && out.scalar_type() == k_cache.scalar_type() &&
               rows2d(out, T, (int64_t)H * vdim), "attn_diff_window: out [T, H vdim]");
   TORCH_CHECK(window >= 0, "attn_diff_window: window");
+  if (short_rows > 0) {
+    // sequences of at most short_rows rows each (decode section): one workgroup per
+    // (sequence, row, key/value head); falls through to the work items if the LDS is too small
+    TORCH_CHECK(short_rows <= 65535 && G <= 65535, "attn_diff_window: short_rows");
+    const int kt = rfqmix::launch_attn_diff_decode(
+        f32, f32p(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), i32p(bt, "block_tables", 0),
+        (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
+        i32p(kv_len, "kv_len", NB), NB, (int)short_rows, gate.data_ptr(), gate.stride(0),
+        out.data_ptr(), out.stride(0), (float)scale, (int)window, (float)lam, (float)eps,
+        (float)out_mult, H, G, dim, vdim, BS, stream());
+    if (kt > 0) return;
+  }
+  if (mfma && !f32 && rfqmix::diff_mfma_ok(dim, vdim, BS)) {
+    // bf16 pages with sizes of the MFMA tiles; 16-byte rows of q and of the pages
+    TORCH_CHECK(reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0 &&
+                reinterpret_cast<uintptr_t>(k_cache.data_ptr()) % 16 == 0 &&
+                reinterpret_cast<uintptr_t>(v_cache.data_ptr()) % 16 == 0,
+                "attn_diff_window: alignment of q and the pages");
+    rfqmix::launch_attn_diff_mfma(
+        f32p(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), i32p(bt, "block_tables", 0),
+        (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
+        i32p(kv_len, "kv_len", NB), i32p(work_seq, "work_seq", W), i32p(work_qblk, "work_qblk", W),
+        W, gate.data_ptr(), gate.stride(0), out.data_ptr(), out.stride(0), (float)scale,
+        (int)window, (float)lam, (float)eps, (float)out_mult, H, G, dim, vdim, BS, stream());
+    return;
+  }
   const bool ok = rfqmix::launch_attn_diff_window(
       f32, f32p(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), i32p(bt, "block_tables", 0),
       (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
@@ -583,6 +618,10 @@ void attn_diff_window(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
       gate.data_ptr(), gate.stride(0), out.data_ptr(), out.stride(0), (float)scale, (int)window,
       (float)lam, (float)eps, (float)out_mult, H, G, dim, vdim, BS, stream());
   TORCH_CHECK(ok, "attn_diff_window: value size too large for the LDS");
+}
+
+bool diff_mfma_ok(int64_t dim, int64_t vdim, int64_t BS) {
+  return rfqmix::diff_mfma_ok((int)dim, (int)vdim, (int)BS);
 }
 
 void conv_act_heads(const Tensor& x, const Tensor& w, const Tensor& state, const Tensor& row_state,
@@ -596,7 +635,7 @@ void conv_act_heads(const Tensor& x, const Tensor& w, const Tensor& state, const
   TORCH_CHECK(state.size(0) % 2 == 0 && state.size(1) == taps - 1 && state.size(2) == C,
               "conv_act_heads: state [2S, taps-1, C]");
   TORCH_CHECK(n_unit >= 0 && dim >= 1 && n_unit * dim <= C, "conv_act_heads: unit heads");
-  TORCH_CHECK((int64_t)C * 4 <= 64 * 1024, "conv_act_heads: too many channels for the LDS");
+  TORCH_CHECK(dim <= 8192 && (C + 255) / 256 <= 65535, "conv_act_heads: sizes");
   TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == C, "conv_act_heads: out [T, C]");
   rfqmix::launch_conv_act_heads(f32, x.data_ptr(), x.stride(0), f32p(w, "w"),
                                 const_cast<float*>(f32p(state, "state")),
@@ -708,7 +747,8 @@ TORCH_LIBRARY(rfq_mix, m) {
   m.def("moe_pair_up(Tensor h, Tensor ids, Tensor w13, Tensor(a!) act) -> ()");
   m.def("residual_add_norm(Tensor(a!) x, Tensor? y1, Tensor? y2, Tensor? shift, Tensor? w, float eps, float offset, Tensor(b!)? out) -> ()");
   m.def("rotary_append(Tensor qkv, Tensor pos, Tensor inv_freq, Tensor slots, Tensor(a!) k_cache, Tensor(b!) v_cache, int H, int G, int maps, int dim, int vdim, Tensor(c!) q_out) -> ()");
-  m.def("attn_diff_window(Tensor q, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor gate, Tensor(a!) out, float scale, int window, float lam, float eps, float out_mult) -> ()");
+  m.def("attn_diff_window(Tensor q, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor gate, Tensor(a!) out, float scale, int window, float lam, float eps, float out_mult, int short_rows, bool mfma) -> ()");
+  m.def("diff_mfma_ok", &diff_mfma_ok);
   m.def("conv_act_heads(Tensor x, Tensor w, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, int n_unit, int dim, float unit_eps, Tensor(b!) out) -> ()");
   m.def("gated_linear_recurrence(Tensor q, Tensor k, Tensor v, Tensor z, Tensor rate, Tensor zbias, float zsign, Tensor? beta, Tensor gate, bool gate_sigmoid, Tensor norm_w, float eps, float q_scale, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor? run_rows, Tensor(b!) out) -> ()");
   m.def("moe_route_topk(Tensor z, Tensor? bias, int top, Tensor(a!) ids, Tensor(b!) weights) -> ()");

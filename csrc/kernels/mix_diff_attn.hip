@@ -191,6 +191,128 @@ __global__ __launch_bounds__(256) void attn_diff_window_kernel(
   }
 }
 
+// ------------------------------------------------------------------ decode rows
+// One workgroup per (sequence, key/value head) and row of the short run: the rep = H / G heads
+// of the group, two maps each, are R = 2 rep score rows over ONE pass through the group's
+// key and value pages (a decode step streams every page once, not once per head).  A wave
+// takes a score row at a time, a lane a key of the tile; the weighted sums of a tile are
+// spread over all threads by (row, value channel).
+// LDS (floats): qs[rep][kw] | Ks[KT][kw + 1] | Vs[KT][vdim] | Ps[R][KT] | acc[R][vdim] |
+//               mrow[R] | lrow[R] | arow[R]
+template <typename T>
+__global__ __launch_bounds__(256) void attn_diff_decode_kernel(
+    const float* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int32_t* __restrict__ block_tables, int maxb, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ q_len, const int32_t* __restrict__ kv_len,
+    const T* __restrict__ gate, int64_t gate_stride, T* __restrict__ out, int64_t out_stride,
+    float scale, int window, float lam, float eps, float out_mult, int H, int G, int dim,
+    int vdim, int BS, int KT) {
+  const int s = blockIdx.x, g = blockIdx.y;
+  const int ql = q_len[s];
+  const int32_t* bt = block_tables + (int64_t)s * maxb;
+  const int rep = H / G, R = 2 * rep, kw = 2 * dim;
+  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6, nw = blockDim.x >> 6;
+  const int nthr = blockDim.x;
+
+  extern __shared__ float lds[];
+  float* qs = lds;
+  float* Ks = qs + rep * kw;
+  float* Vs = Ks + KT * (kw + 1);
+  float* Ps = Vs + KT * vdim;
+  float* acc = Ps + R * KT;
+  float* mrow = acc + R * vdim;
+  float* lrow = mrow + R;
+  float* arow = lrow + R;
+
+  // the rows of a short run one after the other, gridDim.z of them at a time (a decode
+  // step has one row per sequence: a grid over all possible rows would be mostly empty)
+  for (int r = blockIdx.z; r < ql; r += gridDim.z) {
+  const int t = q_start[s] + r;
+  const int p = kv_len[s] - ql + r;                    // position of this row
+  const int jlo = window > 0 ? max(0, p - window + 1) : 0;
+  __syncthreads();                                     // the last row's reads are done
+  for (int x = tid; x < rep * kw; x += nthr) qs[x] = q[((int64_t)t * H + g * rep) * kw + x];
+  for (int x = tid; x < R * vdim; x += nthr) acc[x] = 0.f;
+  for (int x = tid; x < R; x += nthr) {
+    mrow[x] = kNegInfD;
+    lrow[x] = 0.f;
+  }
+
+  for (int jb = jlo; jb <= p; jb += KT) {
+    const int nk = min(KT, p + 1 - jb);
+    __syncthreads();                                   // the last tile's sums are done
+    for (int x = tid; x < nk * kw; x += nthr) {
+      const int jj = x / kw, e = x - jj * kw, j = jb + jj;
+      Ks[jj * (kw + 1) + e] =
+          ldf(k_cache + (((int64_t)bt[j / BS] * G + g) * BS + j % BS) * (int64_t)kw + e);
+    }
+    for (int x = tid; x < nk * vdim; x += nthr) {
+      const int jj = x / vdim, e = x - jj * vdim, j = jb + jj;
+      Vs[x] = ldf(v_cache + (((int64_t)bt[j / BS] * G + g) * BS + j % BS) * (int64_t)vdim + e);
+    }
+    __syncthreads();
+    for (int row = wid; row < R; row += nw) {
+      const float* qv = qs + (row >> 1) * kw + (row & 1) * dim;
+      float mx = kNegInfD;
+      for (int jj = lane; jj < KT; jj += 64) {
+        float a = kNegInfD;
+        if (jj < nk) {
+          const float* kv = Ks + jj * (kw + 1) + (row & 1) * dim;
+          float d0 = 0.f;
+          for (int e = 0; e < dim; ++e) d0 += qv[e] * kv[e];
+          a = d0 * scale;
+        }
+        Ps[row * KT + jj] = a;
+        mx = fmaxf(mx, a);
+      }
+      mx = wave_max(mx);
+      const float mo = mrow[row];
+      const float mn = fmaxf(mo, mx);
+      float sum = 0.f;
+      for (int jj = lane; jj < KT; jj += 64) {
+        const float v = Ps[row * KT + jj];
+        const float e = v == kNegInfD ? 0.f : expf(v - mn);
+        Ps[row * KT + jj] = e;
+        sum += e;
+      }
+      sum = wave_sum(sum);
+      if (lane == 0) {
+        const float alpha = mo == kNegInfD ? 0.f : expf(mo - mn);
+        arow[row] = alpha;
+        lrow[row] = lrow[row] * alpha + sum;
+        mrow[row] = mn;
+      }
+    }
+    __syncthreads();
+    for (int x = tid; x < R * vdim; x += nthr) {
+      const int row = x / vdim, dv = x - row * vdim;
+      float a = acc[x] * arow[row];
+      const float* pr = Ps + row * KT;
+      for (int jj = 0; jj < nk; ++jj) a += pr[jj] * Vs[jj * vdim + dv];
+      acc[x] = a;
+    }
+  }
+  __syncthreads();
+  for (int hr = wid; hr < rep; hr += nw) {
+    const float l0 = lrow[2 * hr], l1 = lrow[2 * hr + 1];
+    const float i0 = l0 > 0.f ? 1.0f / l0 : 0.f, i1 = l1 > 0.f ? lam / l1 : 0.f;
+    float ss = 0.f;
+    for (int dv = lane; dv < vdim; dv += 64) {
+      const float o = acc[(2 * hr) * vdim + dv] * i0 - acc[(2 * hr + 1) * vdim + dv] * i1;
+      ss += o * o;
+    }
+    ss = wave_sum(ss);
+    const int hh = g * rep + hr;
+    const float gl = ldf(gate + (int64_t)t * gate_stride + hh);
+    const float mul = out_mult / sqrtf(ss / (float)vdim + eps) / (1.0f + expf(-gl));
+    for (int dv = lane; dv < vdim; dv += 64) {
+      const float o = acc[(2 * hr) * vdim + dv] * i0 - acc[(2 * hr + 1) * vdim + dv] * i1;
+      stf(out + (int64_t)t * out_stride + (int64_t)hh * vdim + dv, o * mul);
+    }
+  }
+  }
+}
+
 // ------------------------------------------------------------------ launcher
 size_t attn_diff_lds(int vdim) {
   return ((size_t)DQB * (DEC + 1) + (size_t)DKT * (DEC + 1) + 2 * (size_t)DQB * (DKT + 1) +
@@ -226,6 +348,53 @@ bool launch_attn_diff_window(bool f32, const float* q, const void* k_cache, cons
                        kv_len, work_seq, work_qblk, (const bf16_t*)gate, gate_stride, (bf16_t*)out,
                        out_stride, scale, window, lam, eps, out_mult, H, G, dim, vdim, BS);
   return true;
+}
+
+static size_t attn_diff_decode_floats(int rep, int dim, int vdim, int KT) {
+  const int R = 2 * rep, kw = 2 * dim;
+  return (size_t)rep * kw + (size_t)KT * (kw + 1) + (size_t)KT * vdim + (size_t)R * KT +
+         (size_t)R * vdim + 3 * (size_t)R;
+}
+
+// Decode rows: one launch over (sequences, G, up to four rows at a time).  Returns the key tile used (0: the
+// sizes do not fit the LDS; the caller then runs the work-item kernel).
+int launch_attn_diff_decode(bool f32, const float* q, const void* k_cache, const void* v_cache,
+                            const int32_t* bt, int maxb, const int32_t* q_start,
+                            const int32_t* q_len, const int32_t* kv_len, int NA, int max_rows,
+                            const void* gate, int64_t gate_stride, void* out, int64_t out_stride,
+                            float scale, int window, float lam, float eps, float out_mult, int H,
+                            int G, int dim, int vdim, int BS, hipStream_t s) {
+  const int rep = H / G;
+  // the largest key tile whose LDS fits two workgroups per CU, else one (160 KB per CU)
+  int KT = 64;
+  while (KT >= 16 && attn_diff_decode_floats(rep, dim, vdim, KT) * 4 > 80 * 1024) KT >>= 1;
+  if (KT < 16) {
+    KT = 64;
+    while (KT >= 16 && attn_diff_decode_floats(rep, dim, vdim, KT) * 4 > 160 * 1024) KT >>= 1;
+  }
+  if (KT < 16) return 0;
+  if (NA == 0) return KT;
+  const size_t lds = attn_diff_decode_floats(rep, dim, vdim, KT) * 4;
+  static bool attr = false;
+  if (!attr) {
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_diff_decode_kernel<float>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_diff_decode_kernel<bf16_t>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    attr = true;
+  }
+  const dim3 grid(NA, G, max_rows < 4 ? max_rows : 4);
+  if (f32)
+    hipLaunchKernelGGL(attn_diff_decode_kernel<float>, grid, dim3(256), lds, s, q,
+                       (const float*)k_cache, (const float*)v_cache, bt, maxb, q_start, q_len,
+                       kv_len, (const float*)gate, gate_stride, (float*)out, out_stride, scale,
+                       window, lam, eps, out_mult, H, G, dim, vdim, BS, KT);
+  else
+    hipLaunchKernelGGL(attn_diff_decode_kernel<bf16_t>, grid, dim3(256), lds, s, q,
+                       (const bf16_t*)k_cache, (const bf16_t*)v_cache, bt, maxb, q_start, q_len,
+                       kv_len, (const bf16_t*)gate, gate_stride, (bf16_t*)out, out_stride, scale,
+                       window, lam, eps, out_mult, H, G, dim, vdim, BS, KT);
+  return KT;
 }
 
 }  // namespace rfqmix

@@ -100,23 +100,27 @@ __global__ __launch_bounds__(256) void rotary_append_kernel(
 // y[t, c] = silu(sum_j w[c, j] x[t - (taps-1-j), c]); rows before the run come from the
 // sequence's state half, rows before position 0 are zero; the run's last taps - 1 inputs go
 // to the other half.  Then heads [0, n_unit) of `dim` channels become unit vectors.
-// LDS: C floats.
+// A workgroup takes `chunk` channels (a multiple of dim, so no head straddles two) of a row.
+// LDS: chunk floats.
 template <typename T>
 __global__ __launch_bounds__(256) void conv_act_heads_kernel(
     const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
     float* __restrict__ state, const int32_t* __restrict__ row_state,
     const int32_t* __restrict__ row_back, const int32_t* __restrict__ row_fwd,
     const int32_t* __restrict__ pos, float* __restrict__ out, int C, int taps, int slots,
-    int n_unit, int dim, float unit_eps) {
+    int n_unit, int dim, float unit_eps, int chunk) {
   extern __shared__ float ys[];
   const int t = blockIdx.x;
+  const int c0 = blockIdx.y * chunk;
+  const int nc = min(chunk, C - c0);
   const int code = row_state[t], i = row_back[t], f = row_fwd[t], p = pos[t];
   const int K = taps - 1;
   const float* rd = code >= 0 ? state + ((int64_t)((code & 1) * slots + (code >> 1)) * K) * C : nullptr;
   float* wr = code >= 0 ? state + ((int64_t)((1 - (code & 1)) * slots + (code >> 1)) * K) * C : nullptr;
   const T* xr = x + (int64_t)t * x_stride;
   const int n = i + f + 1;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+  for (int cc = threadIdx.x; cc < nc; cc += blockDim.x) {
+    const int c = c0 + cc;
     const float x0 = ldf(xr + c);
     const float* wc = w + (int64_t)c * taps;
     float acc = wc[taps - 1] * x0;
@@ -127,17 +131,23 @@ __global__ __launch_bounds__(256) void conv_act_heads_kernel(
       else continue;
       acc += wc[taps - 1 - dl] * src;
     }
-    ys[c] = acc / (1.0f + expf(-acc));
+    ys[cc] = acc / (1.0f + expf(-acc));
     if (wr != nullptr) {
       if (f < K) wr[(int64_t)(K - 1 - f) * C + c] = x0;
       if (i == 0)
         for (int e = 0; e < K - n; ++e) wr[(int64_t)e * C + c] = rd[(int64_t)(e + n) * C + c];
     }
   }
+  float* o = out + (int64_t)t * C + c0;
+  const int first_head = c0 / dim;
+  const int unit_here = min(max(n_unit - first_head, 0), nc / dim);   // unit heads of this chunk
+  if (unit_here == 0) {                   // every thread re-reads only what it wrote itself
+    for (int cc = threadIdx.x; cc < nc; cc += blockDim.x) o[cc] = ys[cc];
+    return;
+  }
   __syncthreads();
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
-  float* o = out + (int64_t)t * C;
-  for (int hd = wid; hd < n_unit; hd += nw) {
+  for (int hd = wid; hd < unit_here; hd += nw) {
     float ss = 0.f;
     for (int e = lane; e < dim; e += 64) {
       const float v = ys[hd * dim + e];
@@ -147,7 +157,7 @@ __global__ __launch_bounds__(256) void conv_act_heads_kernel(
     const float r = 1.0f / sqrtf(ss + unit_eps);
     for (int e = lane; e < dim; e += 64) o[hd * dim + e] = ys[hd * dim + e] * r;
   }
-  for (int c = n_unit * dim + threadIdx.x; c < C; c += blockDim.x) o[c] = ys[c];
+  for (int cc = unit_here * dim + threadIdx.x; cc < nc; cc += blockDim.x) o[cc] = ys[cc];
 }
 
 // One thread per row: the `top` largest of z + bias (ties to the lower index), weights =
@@ -240,15 +250,20 @@ void launch_conv_act_heads(bool f32, const void* x, int64_t stride, const float*
                            int taps, int slots, int n_unit, int dim, float unit_eps,
                            hipStream_t s) {
   if (T_ == 0) return;
-  const size_t lds = (size_t)C * sizeof(float);          // checked <= 64 KB by the caller
+  // about 1024 channels per workgroup (four per thread), whole heads; rows of few channels
+  // or steps of few rows get smaller chunks so that the grid still fills the chip
+  const int want = (T_ >= 1024 && C >= 4096) ? 1024 : 256;
+  const int chunk = dim * ((want + dim - 1) / dim);
+  const size_t lds = (size_t)chunk * sizeof(float);
+  const dim3 grid(T_, (C + chunk - 1) / chunk);
   if (f32)
-    hipLaunchKernelGGL(conv_act_heads_kernel<float>, dim3(T_), dim3(256), lds, s, (const float*)x,
+    hipLaunchKernelGGL(conv_act_heads_kernel<float>, grid, dim3(256), lds, s, (const float*)x,
                        stride, w, state, row_state, row_back, row_fwd, pos, out, C, taps, slots,
-                       n_unit, dim, unit_eps);
+                       n_unit, dim, unit_eps, chunk);
   else
-    hipLaunchKernelGGL(conv_act_heads_kernel<bf16_t>, dim3(T_), dim3(256), lds, s,
-                       (const bf16_t*)x, stride, w, state, row_state, row_back, row_fwd, pos, out,
-                       C, taps, slots, n_unit, dim, unit_eps);
+    hipLaunchKernelGGL(conv_act_heads_kernel<bf16_t>, grid, dim3(256), lds, s, (const bf16_t*)x,
+                       stride, w, state, row_state, row_back, row_fwd, pos, out, C, taps, slots,
+                       n_unit, dim, unit_eps, chunk);
 }
 
 void launch_moe_route_topk(const float* z, const float* bias, int T_, int E, int top, int32_t* ids,

@@ -226,8 +226,9 @@ def _b_attention(H, G, dim, vdim, window, lens, q_lens, out, name):
     flops = (4.0 * dim + 4.0 * vdim) * H * pairs
     seen = sum(min(n, window + q - 1) for n, q in zip(lens, q_lens))
     nbytes = seen * G * (2 * dim + vdim) * 2 + T * H * (2 * dim * 4 + vdim * 2)
+    short = ops.TALK_DECODE_MAX_ROWS if name == "decode" else 0
     t = _time(lambda: ops.attn_diff_window(q, kc, vc, bt, qs, ql, kl, ws, wq, gate, o, dim ** -0.5,
-                                           window, 0.4, 1e-5, 0.4), reps=5, warm=2)
+                                           window, 0.4, 1e-5, 0.4, short), reps=5, warm=2)
     out[f"attn_diff_window ({name})"] = _entry(t, nbytes, flops)
 
 

@@ -137,7 +137,7 @@ class BilolixLM:
             ids, zeros = self._decode_work(m.dec_q_len.shape[0])
             ops.attn_diff_window(q[:D], kc, vc, m.dec_block_tables, m.dec_q_start, m.dec_q_len,
                                  m.dec_kv_len, ids, zeros, gate[:D], attn[:D], mx.scale, mx.window,
-                                 lw["lam"], eps, keep)
+                                 lw["lam"], eps, keep, short_rows=ops.TALK_DECODE_MAX_ROWS)
         if T > D:
             ops.attn_diff_window(q[D:], kc, vc, m.pf_block_tables, m.pf_q_start, m.pf_q_len,
                                  m.pf_kv_len, m.work_seq, m.work_qblk, gate[D:T], attn[D:T],

@@ -1313,17 +1313,28 @@ def rotary_append(qkv, positions, inv_freq, slot_mapping, k_cache, v_cache, H: i
 
 
 DIFF_QBLK = 32       # queries per work item of attn_diff_window (the scheduler's MIXQ_QBLK)
+DIFF_MFMA = os.environ.get("RFQ_DIFF_MFMA", "1") != "0"     # bf16: MFMA tiles where sizes fit
+
+
+def diff_mfma_ok(dim: int, vdim: int, block: int = 32) -> bool:
+    """Whether the MFMA tiles of attn_diff_window cover these sizes (bf16 pages, GPU)."""
+    return bool(DIFF_MFMA and _native.mix_ops().diff_mfma_ok(dim, vdim, block))
 
 
 def attn_diff_window(q, k_cache, v_cache, block_tables, q_start, q_len, kv_len, work_seq,
                      work_qblk, gate, out, scale: float, window: int, lam: float, eps: float,
-                     out_mult: float):
-    """Work items (sequence, block of DIFF_QBLK queries) as for attn_mixq_prefill; a decode
-    section's sequences are one work item each (block 0)."""
+                     out_mult: float, short_rows: int = 0, mfma: bool | None = None):
+    """Work items (sequence, block of DIFF_QBLK queries) as for attn_mixq_prefill.
+    ``short_rows`` > 0: every sequence has at most that many rows (a decode section); the
+    kernel then runs one workgroup per (sequence, row, key/value head), all heads of the group
+    over one pass through the pages, and the work lists are only the fallback.  bf16 pages
+    whose sizes the MFMA tiles cover run on them unless ``mfma`` is False (the FMA kernel)."""
     if _gpu(q):
         _native.mix_ops().attn_diff_window(q, k_cache, v_cache, block_tables, q_start, q_len,
                                            kv_len, work_seq, work_qblk, gate, out, float(scale),
-                                           int(window), float(lam), float(eps), float(out_mult))
+                                           int(window), float(lam), float(eps), float(out_mult),
+                                           int(short_rows),
+                                           DIFF_MFMA if mfma is None else bool(mfma))
     else:
         ref.attn_diff_window(q, k_cache, v_cache, block_tables, q_start, q_len, kv_len, gate, out,
                              scale, window, lam, eps, out_mult)

@@ -117,7 +117,8 @@ def _paged(k, v, order, device, dtype=torch.float32):
     return kc.to(device), vc.to(device), bt
 
 
-def _attend(device, q, k, v, gate, sections, scale, window, lam, eps, mult, dtype=torch.float32):
+def _attend(device, q, k, v, gate, sections, scale, window, lam, eps, mult, dtype=torch.float32,
+            mfma=None):
     """sections: [(first row, rows)] of ONE sequence of L rows, each run as its own launch with
     everything before it already cached; returns out [L, H vdim]."""
     L, H = q.shape[:2]
@@ -130,7 +131,7 @@ def _attend(device, q, k, v, gate, sections, scale, window, lam, eps, mult, dtyp
                              i32([0], device), i32([n], device), i32([lo + n], device),
                              i32([0] * nblk, device), i32(list(range(nblk)), device),
                              gate[lo:lo + n].to(dtype).to(device), out[lo:lo + n], scale, window,
-                             lam, eps, mult)
+                             lam, eps, mult, 0, mfma)
     return out
 
 
@@ -180,6 +181,52 @@ def test_a_key_at_the_window_edge_stands_out(device, window, decoded):
         got = _attend(device, q.reshape(L, H, 2 * dim), k.reshape(L, G, 2 * dim), v, gate, sections,
                       scale, window, 0.0, eps, 1.0)
         close(got, want, 5e-5)
+        spread = float(got[L - 1, :vdim].double().std())
+        assert (spread < 0.05) == inside, (window, inside, spread)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,dim,vdim", [(4, 2, 32, 32), (2, 1, 64, 128), (8, 2, 128, 64), (3, 3, 64, 64)])
+@pytest.mark.parametrize("window", [0, 1, 31, 32, 33, 100])
+def test_differential_attention_on_mfma_tiles(H, G, dim, vdim, window):
+    """bf16 pages with sizes of the MFMA tiles: prompt portions cut inside pages and query
+    blocks against the dense computation on the same (rounded) keys and values, and against
+    the FMA kernel to within the output's rounding."""
+    assert ops.diff_mfma_ok(dim, vdim)
+    g = torch.Generator().manual_seed(30)
+    L, scale, lam, diff, eps = 200, dim ** -0.5 * 2, 0.37, 0.6, 1e-4
+    q = torch.randn(L, H, 2, dim, generator=g)
+    k = torch.randn(L, G, 2, dim, generator=g).bfloat16().float()
+    v = torch.randn(L, G, vdim, generator=g).bfloat16().float()
+    gate = torch.randn(L, H, generator=g).bfloat16().float()
+    want = oracle.diff_attention(q.double(), k.double(), v.double(), scale, window, lam, diff, eps,
+                                 gate.double()).reshape(L, H * vdim)
+    sections = [(0, 70), (70, 33), (103, 97)]
+    args = (q.reshape(L, H, 2 * dim), k.reshape(L, G, 2 * dim), v, gate, sections, scale, window,
+            lam, eps, 1.0 - diff)
+    got = _attend("cuda", *args, dtype=torch.bfloat16, mfma=True)
+    fma = _attend("cuda", *args, dtype=torch.bfloat16, mfma=False)
+    close(got, want, 6e-3)                                   # bf16 output
+    assert float((got.double() - fma.double()).abs().max()) <= 2.0 ** -7 * float(want.abs().max())
+    assert float((got.double() - fma.double()).abs().mean()) <= 2e-4 * float(want.abs().max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("window", [33, 64, 65])
+def test_mfma_tiles_see_the_window_edge(window):
+    """The standing-out key just inside / just outside the window, on the MFMA tiles."""
+    g = torch.Generator().manual_seed(31)
+    L, H, G, dim, vdim, eps = 140, 2, 1, 32, 32, 1e-6
+    for inside in (True, False):
+        q = torch.randn(L, H, 2, dim, generator=g) * 0.1
+        k = (torch.randn(L, G, 2, dim, generator=g) * 0.1).bfloat16().float()
+        v = torch.randn(L, G, vdim, generator=g).bfloat16().float()
+        j = L - 1 - (window - 1) - (0 if inside else 1)
+        q[L - 1, :, 0] = 3.0
+        k[j, 0, 0] = 3.0
+        v[j, 0] = 100.0
+        got = _attend("cuda", q.reshape(L, H, 2 * dim), k.reshape(L, G, 2 * dim), v, torch.zeros(L, H),
+                      [(0, L)], 1.0, window, 0.0, eps, 1.0, dtype=torch.bfloat16, mfma=True)
         spread = float(got[L - 1, :vdim].double().std())
         assert (spread < 0.05) == inside, (window, inside, spread)
 
