@@ -197,7 +197,7 @@ __global__ __launch_bounds__(256) void attn_diff_window_kernel(
 // key and value pages (a decode step streams every page once, not once per head).  A wave
 // takes a score row at a time, a lane a key of the tile; the weighted sums of a tile are
 // spread over all threads by (row, value channel).
-// LDS (floats): qs[rep][kw] | Ks[KT][kw + 1] | Vs[KT][vdim] | Ps[R][KT] | acc[R][vdim] |
+// LDS (floats): qs[rep][kw] | Ks[KT][kw + 4 or 1] | Vs[KT][vdim] | Ps[R][KT] | acc[R][vdim] |
 //               mrow[R] | lrow[R] | arow[R]
 template <typename T>
 __global__ __launch_bounds__(256) void attn_diff_decode_kernel(
@@ -214,16 +214,55 @@ __global__ __launch_bounds__(256) void attn_diff_decode_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6, nw = blockDim.x >> 6;
   const int nthr = blockDim.x;
 
-  extern __shared__ float lds[];
+  // every region starts 16-byte aligned; with dim a multiple of 4 key rows are read in
+  // 16-byte pieces (row stride kw + 4), else one float at a time (row stride kw + 1)
+  const bool vec = (dim & 3) == 0;
+  const int krs = kw + (vec ? 4 : 1);
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   float* qs = lds;
-  float* Ks = qs + rep * kw;
-  float* Vs = Ks + KT * (kw + 1);
-  float* Ps = Vs + KT * vdim;
+  float* Ks = qs + ((rep * kw + 3) & ~3);
+  float* Vs = Ks + ((KT * krs + 3) & ~3);
+  float* Ps = Vs + ((KT * vdim + 3) & ~3);
   float* acc = Ps + R * KT;
   float* mrow = acc + R * vdim;
   float* lrow = mrow + R;
   float* arow = lrow + R;
 
+  // bf16 pages whose rows are whole 16-byte pieces: `width` values of key row jb + jj from
+  // `cache` to dst[jj * dstride ...] as floats
+  const bool vec8 = sizeof(T) == 2 && (kw & 7) == 0 && (vdim & 7) == 0 && (BS & (BS - 1)) == 0;
+  const int bs_shift = 31 - __builtin_clz(BS);
+  auto stage8 = [&](const T* cache, int width, int dstride, float* dst, int jb, int nk) {
+    const int w8 = width >> 3, total = nk * w8;
+    for (int x0 = tid; x0 < total; x0 += 4 * nthr) {
+      uint4 r[4];
+      int at[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int x = x0 + u * nthr;
+        at[u] = -1;
+        if (x < total) {
+          const int jj = x / w8, c = x - jj * w8, j = jb + jj;
+          const int64_t rowi = ((int64_t)bt[j >> bs_shift] * G + g) * BS + (j & (BS - 1));
+          r[u] = *reinterpret_cast<const uint4*>(cache + rowi * width + c * 8);
+          at[u] = jj * dstride + c * 8;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (at[u] >= 0) {
+          const uint32_t w[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
+          float f[8];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __uint_as_float(w[i] << 16);
+            f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+          }
+          *reinterpret_cast<float4*>(dst + at[u]) = make_float4(f[0], f[1], f[2], f[3]);
+          *reinterpret_cast<float4*>(dst + at[u] + 4) = make_float4(f[4], f[5], f[6], f[7]);
+        }
+    }
+  };
   // the rows of a short run one after the other, gridDim.z of them at a time (a decode
   // step has one row per sequence: a grid over all possible rows would be mostly empty)
   for (int r = blockIdx.z; r < ql; r += gridDim.z) {
@@ -241,15 +280,27 @@ __global__ __launch_bounds__(256) void attn_diff_decode_kernel(
   for (int jb = jlo; jb <= p; jb += KT) {
     const int nk = min(KT, p + 1 - jb);
     __syncthreads();                                   // the last tile's sums are done
-    for (int x = tid; x < nk * kw; x += nthr) {
-      const int jj = x / kw, e = x - jj * kw, j = jb + jj;
-      Ks[jj * (kw + 1) + e] =
-          ldf(k_cache + (((int64_t)bt[j / BS] * G + g) * BS + j % BS) * (int64_t)kw + e);
+    bool staged = false;
+    if constexpr (sizeof(T) == 2) {
+      if (vec8) {
+        // 16-byte pieces (8 values), four in flight per thread before the first is stored
+        stage8(k_cache, kw, krs, Ks, jb, nk);
+        stage8(v_cache, vdim, vdim, Vs, jb, nk);
+        staged = true;
+      }
     }
-    for (int x = tid; x < nk * vdim; x += nthr) {
-      const int jj = x / vdim, e = x - jj * vdim, j = jb + jj;
-      Vs[x] = ldf(v_cache + (((int64_t)bt[j / BS] * G + g) * BS + j % BS) * (int64_t)vdim + e);
+    if (!staged) {
+      for (int jj = wid; jj < nk; jj += nw) {          // a wave per key row: one address per row
+        const int j = jb + jj;
+        const int64_t at = ((int64_t)bt[j / BS] * G + g) * BS + j % BS;
+        const T* kr = k_cache + at * kw;
+        const T* vr = v_cache + at * vdim;
+        for (int e = lane; e < kw; e += 64) Ks[jj * krs + e] = ldf(kr + e);
+        for (int e = lane; e < vdim; e += 64) Vs[jj * vdim + e] = ldf(vr + e);
+      }
     }
+    // the sums below walk the tile four keys at a time: rows past its end count as zeros
+    for (int x = nk * vdim + tid; x < ((nk + 3) & ~3) * vdim; x += nthr) Vs[x] = 0.f;
     __syncthreads();
     for (int row = wid; row < R; row += nw) {
       const float* qv = qs + (row >> 1) * kw + (row & 1) * dim;
@@ -257,9 +308,17 @@ __global__ __launch_bounds__(256) void attn_diff_decode_kernel(
       for (int jj = lane; jj < KT; jj += 64) {
         float a = kNegInfD;
         if (jj < nk) {
-          const float* kv = Ks + jj * (kw + 1) + (row & 1) * dim;
+          const float* kv = Ks + jj * krs + (row & 1) * dim;
           float d0 = 0.f;
-          for (int e = 0; e < dim; ++e) d0 += qv[e] * kv[e];
+          if (vec) {
+            for (int e = 0; e < dim; e += 4) {
+              const float4 q4 = *reinterpret_cast<const float4*>(qv + e);
+              const float4 k4 = *reinterpret_cast<const float4*>(kv + e);
+              d0 += q4.x * k4.x + q4.y * k4.y + q4.z * k4.z + q4.w * k4.w;
+            }
+          } else {
+            for (int e = 0; e < dim; ++e) d0 += qv[e] * kv[e];
+          }
           a = d0 * scale;
         }
         Ps[row * KT + jj] = a;
@@ -284,12 +343,28 @@ __global__ __launch_bounds__(256) void attn_diff_decode_kernel(
       }
     }
     __syncthreads();
-    for (int x = tid; x < R * vdim; x += nthr) {
-      const int row = x / vdim, dv = x - row * vdim;
-      float a = acc[x] * arow[row];
-      const float* pr = Ps + row * KT;
-      for (int jj = 0; jj < nk; ++jj) a += pr[jj] * Vs[jj * vdim + dv];
-      acc[x] = a;
+    // a thread takes a value channel and up to four score rows: a value is read once for all
+    // of them, the weights of four keys in one 16-byte read
+    const int RG = (R + 3) >> 2;
+    for (int x = tid; x < vdim * RG; x += nthr) {
+      const int rg = x / vdim, dv = x - rg * vdim;
+      const int r0 = rg * 4, nr = min(4, R - r0);
+      float a[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = i < nr ? acc[(r0 + i) * vdim + dv] * arow[r0 + i] : 0.f;
+      for (int jj = 0; jj < nk; jj += 4) {
+        const float v0 = Vs[jj * vdim + dv], v1 = Vs[(jj + 1) * vdim + dv];
+        const float v2 = Vs[(jj + 2) * vdim + dv], v3 = Vs[(jj + 3) * vdim + dv];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (i < nr) {
+            const float4 p4 = *reinterpret_cast<const float4*>(Ps + (r0 + i) * KT + jj);
+            a[i] += p4.x * v0 + p4.y * v1 + p4.z * v2 + p4.w * v3;
+          }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (i < nr) acc[(r0 + i) * vdim + dv] = a[i];
     }
   }
   __syncthreads();
@@ -352,8 +427,8 @@ bool launch_attn_diff_window(bool f32, const float* q, const void* k_cache, cons
 
 static size_t attn_diff_decode_floats(int rep, int dim, int vdim, int KT) {
   const int R = 2 * rep, kw = 2 * dim;
-  return (size_t)rep * kw + (size_t)KT * (kw + 1) + (size_t)KT * vdim + (size_t)R * KT +
-         (size_t)R * vdim + 3 * (size_t)R;
+  return (size_t)rep * kw + 4 + (size_t)KT * (kw + 4) + 4 + (size_t)KT * vdim + 4 +
+         (size_t)R * KT + (size_t)R * vdim + 3 * (size_t)R;
 }
 
 // Decode rows: one launch over (sequences, G, up to four rows at a time).  Returns the key tile used (0: the

@@ -5,14 +5,14 @@
 // four waves are (16 queries) x (score map): a wave keeps the online softmax of its map for
 // its 16 query columns and the map's weighted values O_m^T [vdim x 16] in registers.  A key
 // tile is one page: the head group's keys [32][2 dim] go to LDS as they lie in the page, its
-// values are staged transposed, Vt[vdim][32]; the next page's pieces are loaded into
-// registers while the current one is multiplied.
+// values likewise (read back transposed, ds_read_tr16_b64); the next page's pieces are
+// loaded into registers while the current one is multiplied.
 //
 //   S^T[key, query] = K_m[key, :] . Q_m[query, :]    v_mfma_f32_16x16x32_bf16, A = key rows
 //                     from LDS, B = the queries, held in registers as bf16 hi + lo parts (the
 //                     rotated queries arrive in fp32 and are not rounded a second time)
 //   scale, window mask, online softmax per query column in fp32
-//   O^T[dv, query] += Vt[dv, keys] . P^T[keys, query]   A = two 8-byte reads of Vt, B = the
+//   O^T[dv, query] += V^T[dv, keys] . P^T[keys, query]  A = two transposed reads of V, B = the
 //                     weights straight from the score registers, as bf16 hi + lo parts (two
 //                     MFMAs), so the weights keep fp32's precision.  The score tile leaves a
 //                     lane with keys {4g .. 4g+3} of both 16-key halves; the A operand reads
@@ -32,7 +32,6 @@ using rfq::s16x8;
 namespace {
 constexpr int MQB = 32;                 // queries per work item
 constexpr int MBS = 32;                 // keys per tile = page size
-constexpr int VRS = 36;                 // shorts per Vt row (32 keys + 8 bytes)
 constexpr float kNegInfM = -__builtin_huge_valf();
 
 __device__ __forceinline__ void split_bf16(const float* f, s16x8& hi, s16x8& lo) {
@@ -56,6 +55,7 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
     float out_mult, int H, int G) {
   constexpr int dim = 32 * DK, vdim = 16 * DV, kw = 2 * dim;
   constexpr int KRS = kw + 8;            // shorts per key row in LDS (+ 16 bytes)
+  constexpr int VRS = vdim + 8;          // shorts per value row
   const int s = work_seq[blockIdx.x];
   if (s < 0) return;
   const int hh = blockIdx.y;
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   short* Ks = reinterpret_cast<short*>(smem);            // [32][KRS]
-  short* Vt = Ks + MBS * KRS;                            // [vdim][VRS]
+  short* Vs = Ks + MBS * KRS;                            // [32][VRS]
   // after the last tile the same memory holds both maps' sums, fp32 [2][32][vdim] + 64
   float* Os = reinterpret_cast<float*>(smem);
   float* al = Os + 2 * MQB * vdim;
@@ -134,11 +134,10 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
     for (int a = 0; a < NVV; ++a) {
       const int x = tid + a * 256;
       if (x < MBS * vdim / 8) {
-        const int c = x % (vdim / 8), jj = x / (vdim / 8);
+        const int jj = x / (vdim / 8), c = x - jj * (vdim / 8);
         s16x8 v = vreg[a];
         if (jb + jj > plast) v = (s16x8){0, 0, 0, 0, 0, 0, 0, 0};   // rows never written
-#pragma unroll
-        for (int e = 0; e < 8; ++e) Vt[(c * 8 + e) * VRS + jj] = v[e];
+        *reinterpret_cast<s16x8*>(Vs + jj * VRS + c * 8) = v;
       }
     }
     __syncthreads();
@@ -174,24 +173,32 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float e = sc[kt][i] == kNegInfM ? 0.f : expf(sc[kt][i] - mn);
+        const float e = sc[kt][i] == kNegInfM ? 0.f : __expf(sc[kt][i] - mn);
         pv[kt * 4 + i] = e;
         sum += e;
       }
     sum += __shfl_xor(sum, 16, 64);
     sum += __shfl_xor(sum, 32, 64);
-    const float alpha = mrun == kNegInfM ? 0.f : expf(mrun - mn);
+    const float alpha = mrun == kNegInfM ? 0.f : __expf(mrun - mn);
     lrun = lrun * alpha + sum;
     mrun = mn;
     s16x8 phi, plo;
     split_bf16(pv, phi, plo);
+    // the accumulators are rescaled only on pages that moved some column's running maximum
+    // (wave-uniform test; a factor of exactly 1 changes nothing)
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0ull) {
+#pragma unroll
+      for (int m = 0; m < DV; ++m) o[m] *= alpha;
+    }
+    // transposed reads: a 16-lane group takes 4 key rows x 16 value columns, lane `col`
+    // receives its column (keys 4 grp .. 4 grp + 3 of each 16-key half)
+    const short* v0 = Vs + (4 * grp + (col >> 2)) * VRS + 4 * (col & 3);
+    const short* v1 = v0 + 16 * VRS;
 #pragma unroll
     for (int m = 0; m < DV; ++m) {
-      const short* vr = Vt + (m * 16 + col) * VRS + grp * 4;
-      const s16x4 a0 = *reinterpret_cast<const s16x4*>(vr);
-      const s16x4 a1 = *reinterpret_cast<const s16x4*>(vr + 16);
+      const s16x4 a0 = rfq::ds_read_tr16(v0 + 16 * m);
+      const s16x4 a1 = rfq::ds_read_tr16(v1 + 16 * m);
       const s16x8 a = (s16x8){a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-      o[m] *= alpha;
       o[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(phi), o[m], 0, 0, 0);
       o[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(plo), o[m], 0, 0, 0);
     }
@@ -245,7 +252,7 @@ static void launch_diff_mfma_one(const float* q, const void* k_cache, const void
                                  int64_t out_stride, float scale, int window, float lam, float eps,
                                  float out_mult, int H, int G, hipStream_t s) {
   constexpr int dim = 32 * DK, vdim = 16 * DV, kw = 2 * dim;
-  const size_t tiles = (size_t)(MBS * (kw + 8) + vdim * VRS) * 2;
+  const size_t tiles = (size_t)(MBS * (kw + 8) + MBS * (vdim + 8)) * 2;
   const size_t sums = (size_t)(2 * MQB * vdim + 64) * 4;
   const size_t lds = tiles > sums ? tiles : sums;
   static bool attr = false;
