@@ -160,6 +160,88 @@ __global__ __launch_bounds__(256) void conv_act_heads_kernel(
   for (int cc = unit_here * dim + threadIdx.x; cc < nc; cc += blockDim.x) o[cc] = ys[cc];
 }
 
+// Four channels per thread (2 to 4 taps; C, dim, the row stride and the chunk multiples of 4,
+// 16-byte aligned rows): one 8- or 16-byte load per tap row, the four channels' taps as 4 * taps
+// contiguous floats, 16-byte state accesses and stores.
+__device__ __forceinline__ float4 ld4any(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 ld4any(const bf16_t* p) {
+  const uint2 w = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u),
+                     __uint_as_float(w.y << 16), __uint_as_float(w.y & 0xffff0000u));
+}
+
+template <typename T, int TAPS>
+__global__ __launch_bounds__(256) void conv_act_heads_vec_kernel(
+    const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
+    float* __restrict__ state, const int32_t* __restrict__ row_state,
+    const int32_t* __restrict__ row_back, const int32_t* __restrict__ row_fwd,
+    const int32_t* __restrict__ pos, float* __restrict__ out, int C, int, int slots,
+    int n_unit, int dim, float unit_eps, int chunk) {
+  constexpr int taps = TAPS;
+  extern __shared__ __attribute__((aligned(16))) float ys[];
+  const int t = blockIdx.x;
+  const int c0 = blockIdx.y * chunk;
+  const int nc = min(chunk, C - c0);
+  const int code = row_state[t], i = row_back[t], f = row_fwd[t], p = pos[t];
+  const int K = taps - 1;
+  const float* rd = code >= 0 ? state + ((int64_t)((code & 1) * slots + (code >> 1)) * K) * C : nullptr;
+  float* wr = code >= 0 ? state + ((int64_t)((1 - (code & 1)) * slots + (code >> 1)) * K) * C : nullptr;
+  const T* xr = x + (int64_t)t * x_stride;
+  const int n = i + f + 1;
+  for (int cc = threadIdx.x * 4; cc < nc; cc += blockDim.x * 4) {
+    const int c = c0 + cc;
+    const float4 x0 = ld4any(xr + c);
+    float wc[4 * TAPS];                                  // [4][taps], read in 16-byte pieces
+#pragma unroll
+    for (int k = 0; k < TAPS; ++k)
+      *reinterpret_cast<float4*>(wc + 4 * k) = ld4any(w + (int64_t)c * taps + 4 * k);
+    float a0 = wc[taps - 1] * x0.x, a1 = wc[2 * taps - 1] * x0.y;
+    float a2 = wc[3 * taps - 1] * x0.z, a3 = wc[4 * taps - 1] * x0.w;
+#pragma unroll
+    for (int dl = 1; dl < taps; ++dl) {
+      float4 src;
+      if (dl <= i) src = ld4any(xr - (int64_t)dl * x_stride + c);
+      else if (p - dl >= 0 && rd != nullptr) src = ld4any(rd + (int64_t)(K + i - dl) * C + c);
+      else continue;
+      const int k = taps - 1 - dl;
+      a0 += wc[k] * src.x;
+      a1 += wc[taps + k] * src.y;
+      a2 += wc[2 * taps + k] * src.z;
+      a3 += wc[3 * taps + k] * src.w;
+    }
+    *reinterpret_cast<float4*>(ys + cc) =
+        make_float4(a0 / (1.0f + expf(-a0)), a1 / (1.0f + expf(-a1)), a2 / (1.0f + expf(-a2)),
+                    a3 / (1.0f + expf(-a3)));
+    if (wr != nullptr) {
+      if (f < K) *reinterpret_cast<float4*>(wr + (int64_t)(K - 1 - f) * C + c) = x0;
+      if (i == 0)
+        for (int e = 0; e < K - n; ++e)
+          *reinterpret_cast<float4*>(wr + (int64_t)e * C + c) = ld4any(rd + (int64_t)(e + n) * C + c);
+    }
+  }
+  float* o = out + (int64_t)t * C + c0;
+  const int first_head = c0 / dim;
+  const int unit_here = min(max(n_unit - first_head, 0), nc / dim);
+  if (unit_here == 0) {                   // every thread re-reads only what it wrote itself
+    for (int cc = threadIdx.x * 4; cc < nc; cc += blockDim.x * 4)
+      *reinterpret_cast<float4*>(o + cc) = *reinterpret_cast<const float4*>(ys + cc);
+    return;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  for (int hd = wid; hd < unit_here; hd += nw) {
+    float ss = 0.f;
+    for (int e = lane; e < dim; e += 64) {
+      const float v = ys[hd * dim + e];
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float r = 1.0f / sqrtf(ss + unit_eps);
+    for (int e = lane; e < dim; e += 64) o[hd * dim + e] = ys[hd * dim + e] * r;
+  }
+  for (int cc = unit_here * dim + threadIdx.x; cc < nc; cc += blockDim.x) o[cc] = ys[cc];
+}
+
 // One thread per row: the `top` largest of z + bias (ties to the lower index), weights =
 // softmax over the chosen.  E <= 256.
 __global__ __launch_bounds__(64) void moe_route_topk_kernel(
@@ -256,14 +338,30 @@ void launch_conv_act_heads(bool f32, const void* x, int64_t stride, const float*
   const int chunk = dim * ((want + dim - 1) / dim);
   const size_t lds = (size_t)chunk * sizeof(float);
   const dim3 grid(T_, (C + chunk - 1) / chunk);
-  if (f32)
-    hipLaunchKernelGGL(conv_act_heads_kernel<float>, grid, dim3(256), lds, s, (const float*)x,
-                       stride, w, state, row_state, row_back, row_fwd, pos, out, C, taps, slots,
-                       n_unit, dim, unit_eps, chunk);
-  else
-    hipLaunchKernelGGL(conv_act_heads_kernel<bf16_t>, grid, dim3(256), lds, s, (const bf16_t*)x,
-                       stride, w, state, row_state, row_back, row_fwd, pos, out, C, taps, slots,
-                       n_unit, dim, unit_eps, chunk);
+  const bool vec = taps >= 2 && taps <= 4 && C % 4 == 0 && dim % 4 == 0 && stride % 4 == 0 &&
+                   reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(state) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(out) % 16 == 0;
+#define CONV_GO(KERNEL, TT)                                                                     \
+  hipLaunchKernelGGL(KERNEL<TT>, grid, dim3(256), lds, s, (const TT*)x, stride, w, state,      \
+                     row_state, row_back, row_fwd, pos, out, C, taps, slots, n_unit, dim,       \
+                     unit_eps, chunk)
+#define CONV_VEC(TT)                                                                            \
+  do {                                                                                          \
+    if (taps == 2) hipLaunchKernelGGL((conv_act_heads_vec_kernel<TT, 2>), grid, dim3(256), lds, s, (const TT*)x, stride, w, state, row_state, row_back, row_fwd, pos, out, C, taps, slots, n_unit, dim, unit_eps, chunk); \
+    else if (taps == 3) hipLaunchKernelGGL((conv_act_heads_vec_kernel<TT, 3>), grid, dim3(256), lds, s, (const TT*)x, stride, w, state, row_state, row_back, row_fwd, pos, out, C, taps, slots, n_unit, dim, unit_eps, chunk); \
+    else hipLaunchKernelGGL((conv_act_heads_vec_kernel<TT, 4>), grid, dim3(256), lds, s, (const TT*)x, stride, w, state, row_state, row_back, row_fwd, pos, out, C, taps, slots, n_unit, dim, unit_eps, chunk); \
+  } while (0)
+  if (vec) {
+    if (f32) CONV_VEC(float);
+    else CONV_VEC(bf16_t);
+  } else {
+    if (f32) CONV_GO(conv_act_heads_kernel, float);
+    else CONV_GO(conv_act_heads_kernel, bf16_t);
+  }
+#undef CONV_GO
+#undef CONV_VEC
 }
 
 void launch_moe_route_topk(const float* z, const float* bias, int T_, int E, int top, int32_t* ids,
