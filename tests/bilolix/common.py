@@ -64,6 +64,12 @@ ONE_PASS = config([attention(2, 1, 16, 16, 5, 16, dense(16)), gla(2, 16, 16, 2.0
                   loop=(1, 2, 1))
 
 
+# nothing a multiple of 8: width, head sizes, feed-forward widths, vocabulary
+ODD = config([gla(3, 12, 20, 3.0, dense(18)), attention(5, 5, 6, 10, 9, 6, moe(10, 3, 2), scale=0.7, diff=0.45),
+              delta(3, 1, 10, 14, 3, dense(22)), attention(2, 1, 14, 6, 3, 2, None, base=17.0)],
+             vocab=53, width=36, loop=(0, 2, 2))
+
+
 def build(cfg_dict, device="cpu", dtype=torch.float32, seed=0, full=None, ranks=(6, 10), **eng_kw):
     from dataclasses import replace
 

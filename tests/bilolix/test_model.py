@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from . import oracle
-from .common import (NO_LOOP, ONE_PASS, REGS, SMALL, alone, attention, build, check, config, delta,
+from .common import (NO_LOOP, ODD, ONE_PASS, REGS, SMALL, alone, attention, build, check, config, delta,
                      dense, gla, moe, run_schedule, tokens)
 
 DEVICES = ["cpu", pytest.param("cuda:0", marks=pytest.mark.gpu)]
@@ -20,6 +20,23 @@ def test_whole_prompt_and_token_by_token(device, cfg):
     t = tokens(75, cfg["vocab"], 1)
     check(run_schedule(eng, alone(t, [])), cfg, full, {"a": t})
     check(run_schedule(eng, alone(t, [40] + [1] * 35)), cfg, full, {"a": t})
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_sizes_that_are_multiples_of_nothing(device, dtype):
+    """Width 36, odd head counts and sizes, inner ranks of 5 and 7: every product and kernel
+    takes them, in both types, through prompts, portions and decoding."""
+    eng, full = build(ODD, device, dtype=dtype, ranks=(5, 7))
+    t = tokens(70, ODD["vocab"], 4)
+    got = run_schedule(eng, alone(t, [33, 2, 9] + [1] * 26))
+    if dtype == torch.float32:
+        check(got, ODD, full, {"a": t})
+    else:
+        ref = oracle.forward(ODD, full, t)
+        e = sorted(float(((got[("a", p)].double() - ref[p]) - (got[("a", p)].double() - ref[p]).mean())
+                         .pow(2).mean().sqrt() / ref.std()) for p in range(70))
+        assert e[35] < 0.05 and e[-4] < 0.2, e[-6:]
 
 
 @pytest.mark.parametrize("device", DEVICES)
