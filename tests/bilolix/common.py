@@ -19,7 +19,7 @@ def moe(ff, experts, top):
     return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
 
 
-def attention(heads, kv_heads, dim, vdim, window, rot_dims, mlp, scale=0.3, diff=0.6, base=1000.0):
+def attention(heads, kv_heads, dim, vdim, window, rot_dims, mlp, scale=0.3, diff=0.55, base=1000.0):
     m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale,
          "diff": diff, "mask": {"size": window}, "rot": {"dims": rot_dims, "base": base}}
     return {"type": "attention", "mixer": m, "mlp": mlp}

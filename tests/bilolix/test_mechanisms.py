@@ -142,7 +142,7 @@ def test_differential_attention_in_sections(device, H, G, dim, vdim, window):
     """A prompt portion (several query blocks), a short extend and single decoded rows over
     pages that lie in odd order equal the dense computation of the whole sequence."""
     g = torch.Generator().manual_seed(3)
-    L, scale, lam, diff, eps = 150, 0.4, 0.37, 0.6, 1e-4
+    L, scale, lam, diff, eps = 150, 0.4, 0.37, 0.55, 1e-4
     q = torch.randn(L, H, 2, dim, generator=g)
     k = torch.randn(L, G, 2, dim, generator=g)
     v = torch.randn(L, G, vdim, generator=g)
@@ -194,7 +194,7 @@ def test_differential_attention_on_mfma_tiles(H, G, dim, vdim, window):
     the FMA kernel to within the output's rounding."""
     assert ops.diff_mfma_ok(dim, vdim)
     g = torch.Generator().manual_seed(30)
-    L, scale, lam, diff, eps = 200, dim ** -0.5 * 2, 0.37, 0.6, 1e-4
+    L, scale, lam, diff, eps = 200, dim ** -0.5 * 2, 0.37, 0.55, 1e-4
     q = torch.randn(L, H, 2, dim, generator=g)
     k = torch.randn(L, G, 2, dim, generator=g).bfloat16().float()
     v = torch.randn(L, G, vdim, generator=g).bfloat16().float()
