@@ -651,7 +651,8 @@ void gated_linear_recurrence(const Tensor& q, const Tensor& k, const Tensor& v, 
                              const OptT& beta, const Tensor& gate, bool gate_sigmoid,
                              const Tensor& norm_w, double eps, double q_scale, const Tensor& state,
                              const Tensor& row_state, const Tensor& row_back, const Tensor& row_fwd,
-                             const Tensor& pos, const OptT& run_rows, const Tensor& out) {
+                             const Tensor& pos, const OptT& run_rows, const Tensor& out,
+                             bool decay_ready, const OptT& raw) {
   const bool in_f32 = act_f32(q, "gated_linear_recurrence q");
   const bool a_f32 = act_f32(out, "gated_linear_recurrence out");
   TORCH_CHECK(state.dim() == 4 && state.size(0) % 2 == 0,
@@ -689,6 +690,8 @@ void gated_linear_recurrence(const Tensor& q, const Tensor& k, const Tensor& v, 
   a.gate = gate.data_ptr(); a.gs = gate.stride(0); a.gate_sigmoid = gate_sigmoid ? 1 : 0;
   a.norm_w = f32p(norm_w, "norm_w", vdim);
   a.eps = (float)eps; a.q_scale = (float)q_scale;
+  a.decay_ready = decay_ready ? 1 : 0;
+  a.raw = raw.has_value() ? const_cast<float*>(f32p(*raw, "raw", (int64_t)T * H * vdim)) : nullptr;
   a.state = const_cast<float*>(f32p(state, "state"));
   a.row_state = i32p(row_state, "row_state", T); a.row_back = i32p(row_back, "row_back", T);
   a.row_fwd = i32p(row_fwd, "row_fwd", T); a.pos = i32p(pos, "positions", T);
@@ -697,6 +700,17 @@ void gated_linear_recurrence(const Tensor& q, const Tensor& k, const Tensor& v, 
   a.out = out.data_ptr();
   a.T = T; a.H = H; a.rep = H / Hq; a.dim = dim; a.vdim = vdim; a.slots = (int)state.size(0) / 2;
   rfqmix::launch_gated_linrec(in_f32, a_f32, beta.has_value(), a, stream());
+}
+
+void decay_from_logits(const Tensor& z, const Tensor& rate, const Tensor& zbias, double zsign,
+                       int64_t dim) {
+  TORCH_CHECK(z.is_cuda() && z.scalar_type() == at::kFloat && z.dim() == 2 && z.stride(1) == 1 &&
+              dim >= 1 && z.size(1) % dim == 0, "decay_from_logits: z [T, H dim] float32");
+  const int H = (int)(z.size(1) / dim);
+  TORCH_CHECK((z.size(1) + 1023) / 1024 <= 65535, "decay_from_logits: too wide");
+  rfqmix::launch_decay_from_logits(z.data_ptr<float>(), z.stride(0), f32p(rate, "rate", H),
+                                   f32p(zbias, "zbias", z.size(1)), (float)zsign, (int)z.size(0), H,
+                                   (int)dim, stream());
 }
 
 void moe_route_topk(const Tensor& z, const OptT& bias, int64_t top, const Tensor& ids,
@@ -750,7 +764,8 @@ TORCH_LIBRARY(rfq_mix, m) {
   m.def("attn_diff_window(Tensor q, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor gate, Tensor(a!) out, float scale, int window, float lam, float eps, float out_mult, int short_rows, bool mfma) -> ()");
   m.def("diff_mfma_ok", &diff_mfma_ok);
   m.def("conv_act_heads(Tensor x, Tensor w, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, int n_unit, int dim, float unit_eps, Tensor(b!) out) -> ()");
-  m.def("gated_linear_recurrence(Tensor q, Tensor k, Tensor v, Tensor z, Tensor rate, Tensor zbias, float zsign, Tensor? beta, Tensor gate, bool gate_sigmoid, Tensor norm_w, float eps, float q_scale, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor? run_rows, Tensor(b!) out) -> ()");
+  m.def("gated_linear_recurrence(Tensor q, Tensor k, Tensor v, Tensor z, Tensor rate, Tensor zbias, float zsign, Tensor? beta, Tensor gate, bool gate_sigmoid, Tensor norm_w, float eps, float q_scale, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor? run_rows, Tensor(b!) out, bool decay_ready, Tensor(c!)? raw) -> ()");
+  m.def("decay_from_logits(Tensor(a!) z, Tensor rate, Tensor zbias, float zsign, int dim) -> ()");
   m.def("moe_route_topk(Tensor z, Tensor? bias, int top, Tensor(a!) ids, Tensor(b!) weights) -> ()");
   m.def("gelu_rows(Tensor x, Tensor(a!) out) -> ()");
   m.def("moe_pair_down(Tensor act, Tensor ids, Tensor weights, Tensor w2, Tensor? base, Tensor(a!) out) -> ()");
@@ -782,6 +797,7 @@ TORCH_LIBRARY_IMPL(rfq_mix, CUDA, m) {
   m.impl("attn_diff_window", &attn_diff_window);
   m.impl("conv_act_heads", &conv_act_heads);
   m.impl("gated_linear_recurrence", &gated_linear_recurrence);
+  m.impl("decay_from_logits", &decay_from_logits);
   m.impl("moe_route_topk", &moe_route_topk);
   m.impl("gelu_rows", &gelu_rows);
 }

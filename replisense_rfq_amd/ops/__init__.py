@@ -1352,16 +1352,27 @@ def conv_act_heads(x, w, state, row_state, row_back, row_fwd, positions, n_unit:
     return out
 
 
+LINREC_DECAY_ROWS = 128     # steps with more rows form the decays before the scan
+
+
 def gated_linear_recurrence(q, k, v, z, rate, zbias, zsign: float, beta, gate, gate_sigmoid: bool,
                             norm_w, eps: float, q_scale: float, state, row_state, row_back,
                             row_fwd, positions, out, run_rows=None):
     """``run_rows`` (int32): the first row of every run of the step (-1: none); the kernel
-    launches one workgroup per (run, head)."""
+    launches one workgroup per (run, head).  On the GPU a step of more than
+    LINREC_DECAY_ROWS rows first turns ``z`` into the decays IN PLACE with a row-parallel
+    kernel and leaves norm and gate to another one, so that the token-by-token scan holds
+    neither transcendental work nor a reduction over the head."""
     if _gpu(q):
+        ready = q.shape[0] > LINREC_DECAY_ROWS
+        raw = None
+        if ready:
+            _native.mix_ops().decay_from_logits(z, rate, zbias, float(zsign), int(state.shape[2]))
+            raw = torch.empty(out.shape, dtype=torch.float32, device=out.device)
         _native.mix_ops().gated_linear_recurrence(
             q, k, v, z, rate, zbias, float(zsign), beta, gate, bool(gate_sigmoid), norm_w,
             float(eps), float(q_scale), state, row_state, row_back, row_fwd, positions, run_rows,
-            out)
+            out, ready, raw)
     else:
         ref.gated_linear_recurrence(q, k, v, z, rate, zbias, zsign, beta, gate, gate_sigmoid,
                                     norm_w, eps, q_scale, state, row_state, row_back, row_fwd,

@@ -337,12 +337,13 @@ def _scan_inputs(g, T, H, Hq, dim, vdim):
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("H,Hq,dim,vdim", [(2, 2, 32, 64), (3, 3, 16, 24), (1, 1, 7, 5), (2, 1, 64, 32),
                                            (4, 2, 128, 16), (2, 2, 40, 100)])
-@pytest.mark.parametrize("cuts", [[40], [1] * 40, [2, 1, 33, 4], [17, 2, 2, 19]])
+@pytest.mark.parametrize("cuts", [[40], [1] * 40, [2, 1, 33, 4], [17, 2, 2, 19], [150, 3, 1]])
 @pytest.mark.parametrize("mode", ["gla", "delta"])
 def test_linear_recurrence_in_portions(device, H, Hq, dim, vdim, cuts, mode):
     """The recurrence in portions through a state slot with stale contents equals the scan of
     the whole sequence: the decay acts on key channels, the read-out sees the token's own
-    write, the delta rule subtracts what the state already holds for the key."""
+    write, the delta rule subtracts what the state already holds for the key.  (A long portion
+    has its decays formed ahead of the scan on the GPU, short ones inside it.)"""
     g = torch.Generator().manual_seed(8)
     T, S, slot, eps, scale = sum(cuts), 2, 1, 1e-4, dim ** -0.5
     q, k, v, z, gate, beta = _scan_inputs(g, T, H, Hq, dim, vdim)
