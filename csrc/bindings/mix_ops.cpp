@@ -76,7 +76,6 @@ void launch_conv_act_heads(bool, const void*, int64_t, const float*, float*, con
                            int, int, int, float, hipStream_t);
 void launch_moe_route_topk(const float*, const float*, int, int, int, int32_t*, float*, hipStream_t);
 void launch_gelu_rows(bool, const void*, int64_t, void*, int64_t, int, int, hipStream_t);
-size_t attn_diff_lds(int);
 bool diff_mfma_ok(int, int, int);
 bool launch_attn_diff_mfma(const float*, const void*, const void*, const int32_t*, int,
                            const int32_t*, const int32_t*, const int32_t*, const int32_t*,
