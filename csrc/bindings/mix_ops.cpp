@@ -548,7 +548,7 @@ void rotary_append(const Tensor& qkv, const Tensor& pos, const Tensor& inv_freq,
               v_cache.size(2) == k_cache.size(2),
               "rotary_append: k_cache [blocks, G, BS, maps dim], v_cache [blocks, G, BS, vdim]");
   const int nrot = (int)inv_freq.numel();
-  TORCH_CHECK(2 * nrot <= dim, "rotary_append: more rotated dimensions than a map has");
+  TORCH_CHECK(2 * nrot <= dim && dim <= 8192, "rotary_append: more rotated dimensions than a map has");
   TORCH_CHECK(q_out.dim() == 3 && q_out.size(0) == T && q_out.size(1) == H && q_out.size(2) == kw,
               "rotary_append: q_out [T, H, maps dim]");
   const float* fr = nrot > 0 ? f32p(inv_freq, "inv_freq") : nullptr;

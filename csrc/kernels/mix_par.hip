@@ -54,9 +54,18 @@ __global__ __launch_bounds__(256) void rotary_append_kernel(
     const float* __restrict__ inv_freq, int nrot, const int32_t* __restrict__ slots,
     T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G, int maps, int dim, int vdim,
     int BS, int64_t pool_slots, float* __restrict__ q_out) {
+  extern __shared__ float cs[];                      // [nrot] of (cos, sin): one per pair index
   const int t = blockIdx.x;
   const T* row = qkv + (int64_t)t * stride;
   const float p = (float)pos[t];
+  // the angle depends on the pair index only: every head and map reuses the row's sines
+  for (int i = threadIdx.x; i < nrot; i += blockDim.x) {
+    float sn, c;
+    sincosf(p * inv_freq[i], &sn, &c);
+    cs[2 * i] = c;
+    cs[2 * i + 1] = sn;
+  }
+  __syncthreads();
   const int32_t slot = slots[t];
   const bool keep = slot >= 0 && slot < pool_slots;
   const int half = dim / 2 + (dim & 1);              // pairs per map (+ a lone last entry)
@@ -71,9 +80,8 @@ __global__ __launch_bounds__(256) void rotary_append_kernel(
     const bool pair = 2 * i + 1 < dim;
     float u = ldf(src), v = pair ? ldf(src + 1) : 0.f;
     if (i < nrot && pair) {
-      float sn, cs;
-      sincosf(p * inv_freq[i], &sn, &cs);
-      const float a = u * cs - v * sn, b = v * cs + u * sn;
+      const float c = cs[2 * i], sn = cs[2 * i + 1];
+      const float a = u * c - v * sn, b = v * c + u * sn;
       u = a;
       v = b;
     }
@@ -93,6 +101,90 @@ __global__ __launch_bounds__(256) void rotary_append_kernel(
     for (int x = threadIdx.x; x < G * vdim; x += blockDim.x) {
       const int g = x / vdim, e = x - g * vdim;
       v_cache[(((int64_t)(slot / BS) * G + g) * BS + slot % BS) * (int64_t)vdim + e] = vs[x];
+    }
+  }
+}
+
+// Eight entries (four pairs) per thread: dim, vdim and the row stride multiples of 8, 16-byte
+// aligned rows and pages.
+__device__ __forceinline__ void ld8any(const float* p, float* f) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+__device__ __forceinline__ void ld8any(const bf16_t* p, float* f) {
+  const uint4 w = *reinterpret_cast<const uint4*>(p);
+  const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = __uint_as_float(u[i] << 16);
+    f[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+  }
+}
+__device__ __forceinline__ void st8any(float* p, const float* f) {
+  *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(f[4], f[5], f[6], f[7]);
+}
+__device__ __forceinline__ void st8any(bf16_t* p, const float* f) {
+  uint32_t u[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    bf16_t lo, hi;
+    stf(&lo, f[2 * i]);
+    stf(&hi, f[2 * i + 1]);
+    u[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+  }
+  *reinterpret_cast<uint4*>(p) = make_uint4(u[0], u[1], u[2], u[3]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rotary_append_vec_kernel(
+    const T* __restrict__ qkv, int64_t stride, const int32_t* __restrict__ pos,
+    const float* __restrict__ inv_freq, int nrot, const int32_t* __restrict__ slots,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G, int maps, int dim, int vdim,
+    int BS, int64_t pool_slots, float* __restrict__ q_out) {
+  extern __shared__ float cs[];
+  const int t = blockIdx.x;
+  const T* row = qkv + (int64_t)t * stride;
+  const float p = (float)pos[t];
+  for (int i = threadIdx.x; i < nrot; i += blockDim.x) {
+    float sn, c;
+    sincosf(p * inv_freq[i], &sn, &c);
+    cs[2 * i] = c;
+    cs[2 * i + 1] = sn;
+  }
+  __syncthreads();
+  const int32_t slot = slots[t];
+  const bool keep = slot >= 0 && slot < pool_slots;
+  const int d8 = dim >> 3, kw = maps * dim;
+  const int nq8 = H * maps * d8, nk8 = G * maps * d8, nv8 = (G * vdim) >> 3;
+  const int64_t prow = keep ? ((int64_t)(slot / BS) * G) * BS + slot % BS : 0;   // + g * BS per head
+  for (int x = threadIdx.x; x < nq8 + nk8 + nv8; x += blockDim.x) {
+    float f[8];
+    if (x >= nq8 + nk8) {                              // values: a plain copy into the page
+      if (!keep) continue;
+      const int y = (x - nq8 - nk8) * 8, g = y / vdim, e = y - g * vdim;
+      ld8any(row + (int64_t)(H + G) * kw + y, f);
+      st8any(v_cache + (prow + (int64_t)g * BS) * vdim + e, f);
+      continue;
+    }
+    const bool is_q = x < nq8;
+    const int y = is_q ? x : x - nq8;
+    const int hm = y / d8, i0 = (y - hm * d8) * 4;     // (head, map), first pair index
+    const int e = hm * dim + 2 * i0;
+    ld8any(row + (is_q ? 0 : H * kw) + e, f);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i0 + u < nrot) {
+        const float c = cs[2 * (i0 + u)], sn = cs[2 * (i0 + u) + 1];
+        const float a = f[2 * u] * c - f[2 * u + 1] * sn, b = f[2 * u + 1] * c + f[2 * u] * sn;
+        f[2 * u] = a;
+        f[2 * u + 1] = b;
+      }
+    if (is_q) {
+      st8any(q_out + (int64_t)t * H * kw + e, f);
+    } else if (keep) {
+      const int g = hm / maps, off = e - g * kw;
+      st8any(k_cache + (prow + (int64_t)g * BS) * kw + off, f);
     }
   }
 }
@@ -316,14 +408,24 @@ void launch_rotary_append(bool f32, const void* qkv, int64_t stride, const int32
                           void* v_cache, int T_, int H, int G, int maps, int dim, int vdim, int BS,
                           int64_t pool_slots, float* q_out, hipStream_t s) {
   if (T_ == 0) return;
-  if (f32)
-    hipLaunchKernelGGL(rotary_append_kernel<float>, dim3(T_), dim3(256), 0, s, (const float*)qkv,
-                       stride, pos, inv_freq, nrot, slots, (float*)k_cache, (float*)v_cache, H, G,
-                       maps, dim, vdim, BS, pool_slots, q_out);
-  else
-    hipLaunchKernelGGL(rotary_append_kernel<bf16_t>, dim3(T_), dim3(256), 0, s, (const bf16_t*)qkv,
-                       stride, pos, inv_freq, nrot, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, H, G,
-                       maps, dim, vdim, BS, pool_slots, q_out);
+  const size_t lds = (size_t)(2 * nrot + 2) * sizeof(float);     // dim <= 8192: checked by the caller
+  const bool vec = dim % 8 == 0 && vdim % 8 == 0 && stride % 8 == 0 &&
+                   reinterpret_cast<uintptr_t>(qkv) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(v_cache) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(q_out) % 16 == 0;
+#define ROT_GO(KERNEL, TT)                                                                     \
+  hipLaunchKernelGGL(KERNEL<TT>, dim3(T_), dim3(256), lds, s, (const TT*)qkv, stride, pos,    \
+                     inv_freq, nrot, slots, (TT*)k_cache, (TT*)v_cache, H, G, maps, dim, vdim, \
+                     BS, pool_slots, q_out)
+  if (vec) {
+    if (f32) ROT_GO(rotary_append_vec_kernel, float);
+    else ROT_GO(rotary_append_vec_kernel, bf16_t);
+  } else {
+    if (f32) ROT_GO(rotary_append_kernel, float);
+    else ROT_GO(rotary_append_kernel, bf16_t);
+  }
+#undef ROT_GO
 }
 
 void launch_conv_act_heads(bool f32, const void* x, int64_t stride, const float* w, float* state,

@@ -67,15 +67,16 @@ def test_exact_gelu(device):
 # ------------------------------------------------------------------ rotation and pages
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("H,G,dim,vdim,rot", [(4, 2, 16, 8, 8), (3, 1, 10, 6, 10), (2, 2, 8, 8, 0),
-                                              (1, 1, 6, 5, 2), (8, 4, 64, 64, 32)])
-def test_rotation_of_both_maps_and_cache_append(device, H, G, dim, vdim, rot):
+                                              (1, 1, 6, 5, 2), (8, 4, 64, 64, 32), (2, 1, 24, 16, 10)])
+@pytest.mark.parametrize("pad", [5, 0])
+def test_rotation_of_both_maps_and_cache_append(device, H, G, dim, vdim, rot, pad):
     """Each map of each head is rotated on its own leading dimensions, in neighbouring pairs,
     by the row's position; the rest passes unchanged; v is not rotated; k and v land in the
     page and row that the slot names, wherever that page lies."""
     g = torch.Generator().manual_seed(2)
     T, base, blocks = 9, 777.0, 6
     N = (H + G) * 2 * dim + G * vdim
-    wide = torch.randn(T, N + 5, generator=g)
+    wide = torch.randn(T, N + pad, generator=g)          # pad 0: rows the 16-byte kernel takes
     pos = torch.tensor([0, 1, 2, 40, 41, 500, 31, 32, 33])
     slots = torch.tensor([5 * BS + 0, 5 * BS + 1, 2 * BS + 31, 0, 1, -1, 3 * BS + 7, 4 * BS + 30, BS + 2])
     kc = torch.full((blocks, G, BS, 2 * dim), 9.0, device=device)
