@@ -36,7 +36,8 @@ bool launch_attn_mixq_prefill_mfma(const float*, const float*, const void*, cons
                                    const int32_t*, int, void*, int64_t, const float*, const float*,
                                    int, int, int, int, int, int, bool, hipStream_t);
 bool mixq_mfma_ok(int, int, int, int, int);
-void launch_embed_rows(bool, const int32_t*, const void*, float*, int, int, int, hipStream_t);
+void launch_embed_rows(bool, const int32_t*, const void*, float*, int, int, int, float,
+                       hipStream_t);
 void launch_post_norm_add(bool, const void*, int64_t, float*, const float*, float, float, void*,
                           int, int, hipStream_t);
 void launch_rms_norm_rows(bool, bool, const void*, int64_t, const float*, float, float, void*, int,
@@ -66,8 +67,27 @@ void launch_moe_pair_up(bool, const void*, int64_t, const int32_t*, const void*,
 void launch_moe_pair_down(bool, const void*, const int32_t*, const float*, const void*, const void*,
                           int64_t, float*, int, int, int, int, int, hipStream_t);
 void launch_residual_add_norm(bool, float*, const void*, int64_t, bool, const void*, int64_t, bool,
-                              const float*, const float*, float, float, void*, int, int,
+                              const float*, const float*, float, float, void*, int, int, float,
                               hipStream_t);
+bool launch_qk_norm_rotary_append(bool, const void*, int64_t, const float*, const float*,
+                                  const float*, bool, int, float, const int32_t*, const float*, int,
+                                  float, int, int, const int32_t*, void*, void*, int, int, int, int,
+                                  int, int, int, int, int64_t, float*, hipStream_t);
+bool launch_attn_keep_window(bool, const float*, const void*, const void*, int64_t, const int32_t*,
+                             int, const int32_t*, const int32_t*, const int32_t*, const int32_t*,
+                             const int32_t*, int, const float*, const void*, int64_t, void*,
+                             int64_t, float, int, int, bool, int, int, int, int, int, hipStream_t);
+int launch_attn_keep_decode(bool, const float*, const void*, const void*, int64_t, const int32_t*,
+                            int, const int32_t*, const int32_t*, const int32_t*, int, int,
+                            const float*, const void*, int64_t, void*, int64_t, float, int, int,
+                            bool, int, int, int, int, int, hipStream_t);
+bool keep_mfma_ok(int, int, int);
+void launch_attn_keep_mfma(const float*, const void*, const void*, int64_t, const int32_t*, int,
+                           const int32_t*, const int32_t*, const int32_t*, const int32_t*,
+                           const int32_t*, int, const float*, const void*, int64_t, void*, int64_t,
+                           float, int, int, bool, int, int, int, int, int, hipStream_t);
+void launch_xielu_rows(bool, const void*, int64_t, void*, int64_t, int, int, float, float,
+                       hipStream_t);
 void launch_rotary_append(bool, const void*, int64_t, const int32_t*, const float*, int,
                           const int32_t*, void*, void*, int, int, int, int, int, int, int, int64_t,
                           float*, hipStream_t);
@@ -311,13 +331,14 @@ bool rows2d(const Tensor& t, int64_t T, int64_t n) {
   return t.dim() == 2 && t.size(0) == T && t.size(1) == n && t.stride(1) == 1;
 }
 
-void embed_rows(const Tensor& ids, const Tensor& table, const Tensor& out) {
+void embed_rows(const Tensor& ids, const Tensor& table, const Tensor& out, double scale) {
   const bool f32 = act_f32(table, "embed_rows table");
   const int T = (int)ids.numel(), d = (int)table.size(1);
   TORCH_CHECK(table.dim() == 2 && table.is_contiguous(), "embed_rows: table [V, d]");
   TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == d, "embed_rows: out [T, d]");
   rfqmix::launch_embed_rows(f32, i32p(ids, "ids", T), table.data_ptr(),
-                            const_cast<float*>(f32p(out, "out")), T, d, (int)table.size(0), stream());
+                            const_cast<float*>(f32p(out, "out")), T, d, (int)table.size(0),
+                            (float)scale, stream());
 }
 
 void post_norm_add(const Tensor& y, const Tensor& residual, const Tensor& w, double mult, double eps,
@@ -503,7 +524,7 @@ void moe_pair_down(const Tensor& act, const Tensor& ids, const Tensor& weights, 
 
 // ---- parallel-sublayer layers: residual, rotary differential attention, linear recurrences
 void residual_add_norm(const Tensor& x, const OptT& y1, const OptT& y2, const OptT& shift,
-                       const OptT& w, double eps, double offset, const OptT& out) {
+                       const OptT& w, double eps, double offset, const OptT& out, double mult) {
   TORCH_CHECK(x.dim() == 2, "residual_add_norm: x [T, d]");
   const int T = (int)x.size(0), d = (int)x.size(1);
   const void* yp[2] = {nullptr, nullptr};
@@ -528,7 +549,7 @@ void residual_add_norm(const Tensor& x, const OptT& y1, const OptT& y2, const Op
   }
   rfqmix::launch_residual_add_norm(of32, const_cast<float*>(f32p(x, "x")), yp[0], ys[0], yf[0],
                                    yp[1], ys[1], yf[1], optf(shift, "shift", d), optf(w, "w", d),
-                                   (float)eps, (float)offset, op, T, d, stream());
+                                   (float)eps, (float)offset, op, T, d, (float)mult, stream());
 }
 
 void rotary_append(const Tensor& qkv, const Tensor& pos, const Tensor& inv_freq,
@@ -621,6 +642,145 @@ void attn_diff_window(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
 
 bool diff_mfma_ok(int64_t dim, int64_t vdim, int64_t BS) {
   return rfqmix::diff_mfma_ok((int)dim, (int)vdim, (int)BS);
+}
+
+// ---- projection norms + half-split rotation, attention with kept first tokens, xIELU
+void qk_norm_rotary_append(const Tensor& proj, const OptT& bias, const OptT& q_norm_w,
+                           const OptT& k_norm_w, bool norm_all, int64_t k_norm_n, double eps,
+                           const Tensor& pos, const Tensor& inv_freq, double rot_mult,
+                           int64_t q_rot_off, int64_t k_rot_off, const Tensor& slots,
+                           const OptT& k_cache, const OptT& v_cache, int64_t H, int64_t G,
+                           int64_t qw, int64_t kw, int64_t vdim, int64_t v_mode,
+                           const Tensor& q_out) {
+  const bool f32 = act_f32(proj, "qk_norm_rotary_append proj");
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1, "qk_norm_rotary_append: proj [T, N]");
+  const int T = (int)proj.size(0);
+  TORCH_CHECK(H >= 1 && G >= 0 && qw >= 1 && kw >= 1 && vdim >= 0 && v_mode >= 0 && v_mode <= 2,
+              "qk_norm_rotary_append: sizes");
+  const int64_t W = H * qw + G * kw + (v_mode == 0 ? G * vdim : 0);
+  TORCH_CHECK(proj.size(1) >= W, "qk_norm_rotary_append: proj narrower than q | k | v");
+  TORCH_CHECK(v_mode != 1 || vdim == kw, "qk_norm_rotary_append: values that are the keys have their width");
+  const int nrot = (int)inv_freq.numel();
+  TORCH_CHECK(q_rot_off >= 0 && k_rot_off >= 0 && q_rot_off + 2 * nrot <= qw &&
+              (G == 0 || k_rot_off + 2 * nrot <= kw),
+              "qk_norm_rotary_append: the rotated entries lie outside a head");
+  TORCH_CHECK(k_norm_n >= 0 && k_norm_n <= kw && (!norm_all || k_norm_n == kw),
+              "qk_norm_rotary_append: k_norm_n");
+  const int64_t nqw = norm_all ? H * qw : qw, nkw = norm_all ? G * kw : k_norm_n;
+  void *kp = nullptr, *vp = nullptr;
+  int BS = 1;
+  int64_t pool_slots = 0;
+  if (G > 0) {
+    TORCH_CHECK(k_cache.has_value(), "qk_norm_rotary_append: key heads need pages");
+    const Tensor& kc = *k_cache;
+    TORCH_CHECK(kc.is_cuda() && kc.scalar_type() == proj.scalar_type() && kc.is_contiguous() &&
+                kc.dim() == 4 && kc.size(1) == G && kc.size(3) == kw,
+                "qk_norm_rotary_append: k_cache [blocks, G, BS, kw]");
+    kp = kc.data_ptr();
+    BS = (int)kc.size(2);
+    pool_slots = kc.size(0) * kc.size(2);
+    if (v_mode != 2) {
+      TORCH_CHECK(v_cache.has_value(), "qk_norm_rotary_append: values need pages");
+      const Tensor& vc = *v_cache;
+      TORCH_CHECK(vc.is_cuda() && vc.scalar_type() == proj.scalar_type() && vc.is_contiguous() &&
+                  vc.dim() == 4 && vc.size(0) == kc.size(0) && vc.size(1) == G &&
+                  vc.size(2) == kc.size(2) && vc.size(3) == vdim,
+                  "qk_norm_rotary_append: v_cache [blocks, G, BS, vdim]");
+      vp = vc.data_ptr();
+    }
+  }
+  TORCH_CHECK(q_out.dim() == 3 && q_out.size(0) == T && q_out.size(1) == H && q_out.size(2) == qw,
+              "qk_norm_rotary_append: q_out [T, H, qw]");
+  const float* fr = nrot > 0 ? f32p(inv_freq, "inv_freq") : nullptr;
+  const bool ok = rfqmix::launch_qk_norm_rotary_append(
+      f32, proj.data_ptr(), proj.stride(0), optf(bias, "bias", W), optf(q_norm_w, "q_norm_w", nqw),
+      (G > 0 && k_norm_w.has_value()) ? f32p(*k_norm_w, "k_norm_w", nkw) : nullptr, norm_all,
+      (int)k_norm_n, (float)eps, i32p(pos, "positions", T), fr, nrot, (float)rot_mult,
+      (int)q_rot_off, (int)k_rot_off, i32p(slots, "slots", T), kp, vp, T, (int)H, (int)G, (int)qw,
+      (int)kw, (int)vdim, (int)v_mode, BS, pool_slots, const_cast<float*>(f32p(q_out, "q_out")),
+      stream());
+  TORCH_CHECK(ok, "qk_norm_rotary_append: a row does not fit the LDS");
+}
+
+void attn_keep_window(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, int64_t vdim,
+                      const Tensor& bt, const Tensor& q_start, const Tensor& q_len,
+                      const Tensor& kv_len, const Tensor& work_seq, const Tensor& work_qblk,
+                      const OptT& head_bias, const OptT& gate, const Tensor& out, double scale,
+                      int64_t window, int64_t keep_first, bool sigmoid, int64_t short_rows,
+                      bool mfma) {
+  const bool f32 = act_f32(k_cache, "attn_keep_window k_cache");
+  TORCH_CHECK(q.dim() == 3, "attn_keep_window: q [T, H, E]");
+  const int T = (int)q.size(0), H = (int)q.size(1), E = (int)q.size(2);
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.is_contiguous() &&
+              v_cache.is_contiguous() && v_cache.is_cuda() &&
+              v_cache.scalar_type() == k_cache.scalar_type() && k_cache.size(3) == E &&
+              v_cache.size(1) == k_cache.size(1) && v_cache.size(0) == k_cache.size(0) &&
+              v_cache.size(2) == k_cache.size(2) && vdim >= 1 && v_cache.size(3) >= vdim,
+              "attn_keep_window: k_cache [blocks, G, BS, E], v_cache [blocks, G, BS, >= vdim]");
+  const int G = (int)k_cache.size(1), BS = (int)k_cache.size(2);
+  const int64_t vrs = v_cache.size(3);
+  TORCH_CHECK(G >= 1 && H % G == 0 && H <= 65535, "attn_keep_window: H a multiple of G");
+  const int NB = (int)q_len.numel(), W = (int)work_seq.numel();
+  TORCH_CHECK(bt.dim() == 2 && bt.size(0) == NB, "attn_keep_window: block_tables [NB, maxb]");
+  TORCH_CHECK(work_qblk.numel() >= W, "attn_keep_window: work lists");
+  TORCH_CHECK(!sigmoid || head_bias.has_value(), "attn_keep_window: sigmoid weights need a bias");
+  const void* gp = nullptr;
+  int64_t gs = 0;
+  if (gate.has_value()) {
+    TORCH_CHECK(gate->is_cuda() && gate->scalar_type() == k_cache.scalar_type() &&
+                rows2d(*gate, T, H), "attn_keep_window: gate [T, H] in the cache's type");
+    gp = gate->data_ptr();
+    gs = gate->stride(0);
+  }
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == k_cache.scalar_type() &&
+              rows2d(out, T, (int64_t)H * vdim), "attn_keep_window: out [T, H vdim]");
+  TORCH_CHECK(window >= 0 && keep_first >= 0, "attn_keep_window: window, keep_first");
+  const float* hb = optf(head_bias, "head_bias", H);
+  const bool tiles = mfma && !f32 && rfqmix::keep_mfma_ok(E, (int)vdim, BS) && vrs % 8 == 0 &&
+                     reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(k_cache.data_ptr()) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(v_cache.data_ptr()) % 16 == 0;
+  if (short_rows > 0 && !tiles) {
+    // sequences of at most short_rows rows each (decode section): one workgroup per
+    // (sequence, key/value head); falls through to the work items if the LDS is too small
+    TORCH_CHECK(short_rows <= 65535 && G <= 65535, "attn_keep_window: short_rows");
+    const int kt = rfqmix::launch_attn_keep_decode(
+        f32, f32p(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), vrs, i32p(bt, "block_tables", 0),
+        (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
+        i32p(kv_len, "kv_len", NB), NB, (int)short_rows, hb, gp, gs, out.data_ptr(), out.stride(0),
+        (float)scale, (int)window, (int)keep_first, sigmoid, H, G, E, (int)vdim, BS, stream());
+    if (kt > 0) return;
+  }
+  if (tiles) {
+    rfqmix::launch_attn_keep_mfma(
+        f32p(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), vrs, i32p(bt, "block_tables", 0),
+        (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
+        i32p(kv_len, "kv_len", NB), i32p(work_seq, "work_seq", W), i32p(work_qblk, "work_qblk", W),
+        W, hb, gp, gs, out.data_ptr(), out.stride(0), (float)scale, (int)window, (int)keep_first,
+        sigmoid, H, G, E, (int)vdim, BS, stream());
+    return;
+  }
+  const bool ok = rfqmix::launch_attn_keep_window(
+      f32, f32p(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), vrs, i32p(bt, "block_tables", 0),
+      (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
+      i32p(kv_len, "kv_len", NB), i32p(work_seq, "work_seq", W), i32p(work_qblk, "work_qblk", W), W,
+      hb, gp, gs, out.data_ptr(), out.stride(0), (float)scale, (int)window, (int)keep_first,
+      sigmoid, H, G, E, (int)vdim, BS, stream());
+  TORCH_CHECK(ok, "attn_keep_window: value size too large for the LDS");
+}
+
+bool keep_mfma_ok(int64_t E, int64_t vdim, int64_t BS) {
+  return rfqmix::keep_mfma_ok((int)E, (int)vdim, (int)BS);
+}
+
+void xielu_rows(const Tensor& x, double ap, double an, const Tensor& out) {
+  const bool f32 = act_f32(x, "xielu_rows x");
+  TORCH_CHECK(x.dim() == 2 && out.dim() == 2 && out.sizes() == x.sizes() && x.stride(1) == 1 &&
+              out.stride(1) == 1 && out.is_cuda() && out.scalar_type() == x.scalar_type(),
+              "xielu_rows: x, out [T, F] of one type");
+  TORCH_CHECK((x.size(1) + 255) / 256 <= 65535, "xielu_rows: F too large");
+  rfqmix::launch_xielu_rows(f32, x.data_ptr(), x.stride(0), out.data_ptr(), out.stride(0),
+                            (int)x.size(0), (int)x.size(1), (float)ap, (float)an, stream());
 }
 
 void conv_act_heads(const Tensor& x, const Tensor& w, const Tensor& state, const Tensor& row_state,
@@ -748,7 +908,7 @@ TORCH_LIBRARY(rfq_mix, m) {
   m.def("mixq_mfma_ok", &mixq_mfma_ok);
   m.def("latent_mfma_ok", &latent_mfma_ok);
   m.def("attn_latent_mfma(Tensor q, Tensor pool, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor(a!) out, Tensor? sink, float scale) -> ()");
-  m.def("embed_rows(Tensor ids, Tensor table, Tensor(a!) out) -> ()");
+  m.def("embed_rows(Tensor ids, Tensor table, Tensor(a!) out, float scale) -> ()");
   m.def("post_norm_add(Tensor y, Tensor(a!) residual, Tensor w, float mult, float eps, Tensor(b!)? copy) -> ()");
   m.def("rms_norm_rows(Tensor x, Tensor w, float eps, float offset, Tensor(a!) out) -> ()");
   m.def("latent_norm_append(Tensor x, Tensor w, float eps, Tensor slots, Tensor(a!) pool) -> ()");
@@ -758,10 +918,14 @@ TORCH_LIBRARY(rfq_mix, m) {
   m.def("wkv_recurrence(Tensor r, Tensor k, Tensor v, Tensor zw, Tensor w0, Tensor u, Tensor gate, Tensor norm_w, float eps, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor? run_rows, Tensor(b!) out) -> ()");
   m.def("moe_route_grouped(Tensor z, Tensor correction, int top, int groups, int keep, Tensor(a!) ids, Tensor(b!) weights) -> ()");
   m.def("moe_pair_up(Tensor h, Tensor ids, Tensor w13, Tensor(a!) act) -> ()");
-  m.def("residual_add_norm(Tensor(a!) x, Tensor? y1, Tensor? y2, Tensor? shift, Tensor? w, float eps, float offset, Tensor(b!)? out) -> ()");
+  m.def("residual_add_norm(Tensor(a!) x, Tensor? y1, Tensor? y2, Tensor? shift, Tensor? w, float eps, float offset, Tensor(b!)? out, float mult) -> ()");
   m.def("rotary_append(Tensor qkv, Tensor pos, Tensor inv_freq, Tensor slots, Tensor(a!) k_cache, Tensor(b!) v_cache, int H, int G, int maps, int dim, int vdim, Tensor(c!) q_out) -> ()");
   m.def("attn_diff_window(Tensor q, Tensor k_cache, Tensor v_cache, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor gate, Tensor(a!) out, float scale, int window, float lam, float eps, float out_mult, int short_rows, bool mfma) -> ()");
   m.def("diff_mfma_ok", &diff_mfma_ok);
+  m.def("qk_norm_rotary_append(Tensor proj, Tensor? bias, Tensor? q_norm_w, Tensor? k_norm_w, bool norm_all, int k_norm_n, float eps, Tensor pos, Tensor inv_freq, float rot_mult, int q_rot_off, int k_rot_off, Tensor slots, Tensor(a!)? k_cache, Tensor(b!)? v_cache, int H, int G, int qw, int kw, int vdim, int v_mode, Tensor(c!) q_out) -> ()");
+  m.def("attn_keep_window(Tensor q, Tensor k_cache, Tensor v_cache, int vdim, Tensor bt, Tensor q_start, Tensor q_len, Tensor kv_len, Tensor work_seq, Tensor work_qblk, Tensor? head_bias, Tensor? gate, Tensor(a!) out, float scale, int window, int keep_first, bool sigmoid, int short_rows, bool mfma) -> ()");
+  m.def("keep_mfma_ok", &keep_mfma_ok);
+  m.def("xielu_rows(Tensor x, float ap, float an, Tensor(a!) out) -> ()");
   m.def("conv_act_heads(Tensor x, Tensor w, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, int n_unit, int dim, float unit_eps, Tensor(b!) out) -> ()");
   m.def("gated_linear_recurrence(Tensor q, Tensor k, Tensor v, Tensor z, Tensor rate, Tensor zbias, float zsign, Tensor? beta, Tensor gate, bool gate_sigmoid, Tensor norm_w, float eps, float q_scale, Tensor(a!) state, Tensor row_state, Tensor row_back, Tensor row_fwd, Tensor pos, Tensor? run_rows, Tensor(b!) out, bool decay_ready, Tensor(c!)? raw) -> ()");
   m.def("decay_from_logits(Tensor(a!) z, Tensor rate, Tensor zbias, float zsign, int dim) -> ()");
@@ -794,6 +958,9 @@ TORCH_LIBRARY_IMPL(rfq_mix, CUDA, m) {
   m.impl("residual_add_norm", &residual_add_norm);
   m.impl("rotary_append", &rotary_append);
   m.impl("attn_diff_window", &attn_diff_window);
+  m.impl("qk_norm_rotary_append", &qk_norm_rotary_append);
+  m.impl("attn_keep_window", &attn_keep_window);
+  m.impl("xielu_rows", &xielu_rows);
   m.impl("conv_act_heads", &conv_act_heads);
   m.impl("gated_linear_recurrence", &gated_linear_recurrence);
   m.impl("decay_from_logits", &decay_from_logits);

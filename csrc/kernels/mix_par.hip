@@ -1,6 +1,6 @@
 // Row kernels of parallel-sublayer layers and their mixers' pre-processing:
 //
-//   residual_add_norm   x += y1 + y2 + shift (fp32 stream), then h = rms(x) (w + offset) for
+//   residual_add_norm   x += mult (y1 + y2) + shift (fp32 stream), then h = rms(x) (w + offset) for
 //                       the next layer: one kernel per layer boundary
 //   rotary_append       interleaved-pair rotation of the leading dimensions of every score
 //                       map of q and k; k and v into their pages, q out in fp32
@@ -19,21 +19,22 @@ __device__ __forceinline__ float ld_any(const void* p, bool f32, int64_t i) {
   return f32 ? static_cast<const float*>(p)[i] : ldf(static_cast<const bf16_t*>(p) + i);
 }
 
-// x[t] += y1[t] + y2[t] + shift; out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * (w + offset).
+// x[t] += mult (y1[t] + y2[t]) + shift; out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * (w + offset).
 // y1, y2, shift and (w, out) are each optional; y1 / y2 are fp32 or bf16 (flags).
 template <typename TO>
 __global__ __launch_bounds__(256) void residual_add_norm_kernel(
     float* __restrict__ x, const void* __restrict__ y1, int64_t y1_stride, bool y1_f32,
     const void* __restrict__ y2, int64_t y2_stride, bool y2_f32, const float* __restrict__ shift,
-    const float* __restrict__ w, float eps, float offset, TO* __restrict__ out, int d) {
+    const float* __restrict__ w, float eps, float offset, TO* __restrict__ out, int d, float mult) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   float* xr = x + (int64_t)t * d;
   float ss = 0.f;
   for (int c = threadIdx.x; c < d; c += blockDim.x) {
-    float v = xr[c];
-    if (y1 != nullptr) v += ld_any(y1, y1_f32, (int64_t)t * y1_stride + c);
-    if (y2 != nullptr) v += ld_any(y2, y2_f32, (int64_t)t * y2_stride + c);
+    float y = 0.f;
+    if (y1 != nullptr) y += ld_any(y1, y1_f32, (int64_t)t * y1_stride + c);
+    if (y2 != nullptr) y += ld_any(y2, y2_f32, (int64_t)t * y2_stride + c);
+    float v = xr[c] + y * mult;
     if (shift != nullptr) v += shift[c];
     xr[c] = v;
     ss += v * v;
@@ -393,14 +394,14 @@ __global__ __launch_bounds__(256) void gelu_rows_kernel(const T* __restrict__ x,
 void launch_residual_add_norm(bool out_f32, float* x, const void* y1, int64_t y1s, bool y1f,
                               const void* y2, int64_t y2s, bool y2f, const float* shift,
                               const float* w, float eps, float offset, void* out, int T_, int d,
-                              hipStream_t s) {
+                              float mult, hipStream_t s) {
   if (T_ == 0) return;
   if (out_f32)
     hipLaunchKernelGGL(residual_add_norm_kernel<float>, dim3(T_), dim3(256), 0, s, x, y1, y1s, y1f,
-                       y2, y2s, y2f, shift, w, eps, offset, (float*)out, d);
+                       y2, y2s, y2f, shift, w, eps, offset, (float*)out, d, mult);
   else
     hipLaunchKernelGGL(residual_add_norm_kernel<bf16_t>, dim3(T_), dim3(256), 0, s, x, y1, y1s,
-                       y1f, y2, y2s, y2f, shift, w, eps, offset, (bf16_t*)out, d);
+                       y1f, y2, y2s, y2f, shift, w, eps, offset, (bf16_t*)out, d, mult);
 }
 
 void launch_rotary_append(bool f32, const void* qkv, int64_t stride, const int32_t* pos,

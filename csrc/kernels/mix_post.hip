@@ -12,13 +12,13 @@ namespace rfqmix {
 template <typename T>
 __global__ __launch_bounds__(256) void embed_rows_kernel(
     const int32_t* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out, int d,
-    int vocab) {
+    int vocab, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const T* row = table + (int64_t)id * d;
   float* o = out + (int64_t)t * d;
-  for (int c = threadIdx.x; c < d; c += blockDim.x) o[c] = ldf(row + c);
+  for (int c = threadIdx.x; c < d; c += blockDim.x) o[c] = ldf(row + c) * scale;
 }
 
 // residual[t] += mult * y[t] / sqrt(mean(y[t]^2) + eps) * (1 + w); copy (nullable) receives
@@ -107,14 +107,14 @@ __global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ x, flo
 
 // ------------------------------------------------------------------ launchers
 void launch_embed_rows(bool f32, const int32_t* ids, const void* table, float* out, int T, int d,
-                       int vocab, hipStream_t s) {
+                       int vocab, float scale, hipStream_t s) {
   if (T == 0) return;
   if (f32)
     hipLaunchKernelGGL(embed_rows_kernel<float>, dim3(T), dim3(256), 0, s, ids,
-                       (const float*)table, out, d, vocab);
+                       (const float*)table, out, d, vocab, scale);
   else
     hipLaunchKernelGGL(embed_rows_kernel<bf16_t>, dim3(T), dim3(256), 0, s, ids,
-                       (const bf16_t*)table, out, d, vocab);
+                       (const bf16_t*)table, out, d, vocab, scale);
 }
 
 void launch_post_norm_add(bool y_f32, const void* y, int64_t y_stride, float* residual,

@@ -61,6 +61,9 @@ class LayeredKVCache:
                          latent holds that layer's pool (the same tensor);
       diff_attention     K pool ``[num_blocks, G, block, 2 dim]`` (both score maps of a
                          key head side by side) and V pool ``[num_blocks, G, block, vdim]``;
+      window_attention   K and V pools like ``attention``;
+      rope_latent_attention   like ``latent_attention`` with rows ``[latent | rotated key
+                         part]``, ``kv_rank + rot_dim`` wide;
       wkv, gla, channel_delta   no pages.
     Per-sequence state lives in slots; a sequence owns one while it runs (native core).  Every
     state pool is double buffered: a step reads half ``gen & 1`` of the slot and writes the
@@ -68,7 +71,8 @@ class LayeredKVCache:
     convolutions' last inputs ``[L, 2 sublayers, 2 * slots, taps - 1, d]`` fp32;
     ``layer_state[i]``: name -> ``[2 * slots, ...]`` fp32 for what ``cfg.state_shapes(i)``
     lists (a wkv layer's matrices and its previous input row; a gla or channel_delta
-    layer's matrices, and the convolutions' last inputs)."""
+    layer's matrices, and the convolutions' last inputs; with ``cfg.token_shift`` every
+    layer's previous normed input row)."""
 
     def __init__(self, cfg, num_blocks: int, device, num_slots: int, block_size: int = 32,
                  dtype=torch.bfloat16, prefix_cache: bool = False):
@@ -87,11 +91,14 @@ class LayeredKVCache:
             elif m.kind == "diff_attention":
                 self.k.append(mk((num_blocks, m.kv_heads, block_size, 2 * m.dim), dtype=dtype, device=device))
                 self.v.append(mk((num_blocks, m.kv_heads, block_size, m.vdim), dtype=dtype, device=device))
-            elif m.kind == "latent_attention":
+            elif m.kind == "window_attention":
+                self.k.append(mk((num_blocks, m.kv_heads, block_size, m.dim), dtype=dtype, device=device))
+                self.v.append(mk((num_blocks, m.kv_heads, block_size, m.vdim), dtype=dtype, device=device))
+            elif m.kind in ("latent_attention", "rope_latent_attention"):
                 if m.kv_from >= 0 and len(runs) != cfg.n_layers:
                     raise ValueError("a layer that reads another layer's latent cannot be looped")
                 pool = self.k[m.kv_from] if m.kv_from >= 0 else \
-                    mk((num_blocks, 1, block_size, m.kv_rank), dtype=dtype, device=device)
+                    mk((num_blocks, 1, block_size, m.kv_rank + m.rot_dim), dtype=dtype, device=device)
                 self.k.append(pool)
                 self.v.append(pool)
             else:

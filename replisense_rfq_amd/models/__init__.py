@@ -16,4 +16,8 @@ def layered_model_class(architecture: str):
         from .bilolix import BilolixLM
 
         return BilolixLM
+    if architecture == "Nutitar":
+        from .nutitar import NutitarLM
+
+        return NutitarLM
     raise KeyError(f"no model class for architecture {architecture!r}")

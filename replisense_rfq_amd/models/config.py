@@ -105,7 +105,19 @@ class MixerSpec:
     ``gla``: ``heads`` recurrent heads with a ``dim`` x ``vdim`` state and a decay per key
     channel, sigmoid(z)^(1 / ``tau``).
     ``channel_delta``: the gated delta rule on such states; queries and keys have
-    ``kv_heads`` heads, and q, k, v pass a causal convolution of ``conv`` taps."""
+    ``kv_heads`` heads, and q, k, v pass a causal convolution of ``conv`` taps.
+    ``rope_latent_attention``: latent attention whose heads also hold ``rot_dim`` rotated
+    query dimensions that meet ONE rotated key part shared by all heads; a token caches
+    its latent and that key part (``kv_rank + rot_dim`` numbers); softmax with a sink and a
+    sigmoid output gate per head; ``kv_from`` as for ``latent_attention``.
+    ``window_attention``: grouped heads with ``qk_norm`` over each head (``head``) or over the
+    whole projection (``all``), half-split rotation of the first ``rot_dims`` dimensions,
+    position i sees j <= i with i - j < ``window`` or j < ``keep_first`` (window 0: plain
+    causal); ``weights`` = ``softmax`` or ``sigmoid`` (unnormalised, with a per-head bias);
+    ``bias``: the projections have biases; ``v_is_k``: the values are the keys as projected.
+    The rotating kinds take their frequencies from ``rot_base`` and ``rot_scaling``: () for
+    none, ("yarn", factor, original, fast, slow) or ("banded", factor, original, low,
+    high)."""
     kind: str = "attention"
     heads: int = 4
     kv_heads: int = 2
@@ -122,6 +134,13 @@ class MixerSpec:
     diff: float = 0.0
     tau: float = 1.0
     conv: int = 0
+    rot_dim: int = 0
+    rot_scaling: tuple = ()
+    keep_first: int = 0
+    qk_norm: str = ""
+    weights: str = "softmax"
+    bias: bool = False
+    v_is_k: bool = False
 
     @property
     def group(self) -> int:
@@ -135,7 +154,8 @@ class MlpSpec:
     neighbouring experts (groups = 0: no limit), plus a shared expert of width
     ``shared_ff`` (0: none); ``router`` = ``softmax_top``: the ``top`` largest router logits
     (with a bias), weighted by the softmax over the chosen logits only.  ``gelu``: up
-    projection, exact gelu, down projection."""
+    projection, exact gelu, down projection.  ``xielu``: up projection, a quadratic / exponential
+    unit with two learned numbers, down projection."""
     kind: str = "dense"
     ff: int = 256
     limit: float = 7.0
@@ -175,6 +195,9 @@ class LayeredConfig:
     # has cache pages and state of its own
     loop: tuple = (0, 0, 1)
     gate_rank: int = 16             # channel_delta layers of seeded models (output gate's inner size)
+    # every layer's mixer reads h + (h' - h) * shift, h' the previous token's normed input
+    # (one row of per-sequence state per layer)
+    token_shift: bool = False
 
     @property
     def n_layers(self) -> int:
@@ -217,6 +240,13 @@ class LayeredConfig:
             elif m.kind == "diff_attention":
                 n += d * (2 * m.dim * (m.heads + m.kv_heads) + m.kv_heads * m.vdim + m.heads)
                 n += m.heads * m.vdim * d
+            elif m.kind == "rope_latent_attention":
+                n += d * m.heads * (m.dim + m.rot_dim + 1) + m.heads * m.vdim * d
+                n += m.kv_rank * m.heads * (m.dim + m.vdim)
+                n += d * (m.kv_rank + m.rot_dim) if m.kv_from < 0 else 0
+            elif m.kind == "window_attention":
+                n += d * (m.heads * m.dim + m.kv_heads * (m.dim + (0 if m.v_is_k else m.vdim)))
+                n += m.heads * m.vdim * d
             elif m.kind == "gla":
                 n += 2 * d * m.heads * (m.dim + m.vdim) + m.heads * m.vdim * d
                 n += self.decay_rank * (d + m.heads * m.dim)
@@ -229,7 +259,7 @@ class LayeredConfig:
             if f is not None and f.kind == "moe":
                 n += 3 * d * (f.ff * f.experts + f.shared_ff) + d * f.experts
             elif f is not None:
-                n += (2 if f.kind == "gelu" else 3) * d * f.ff
+                n += (2 if f.kind in ("gelu", "xielu") else 3) * d * f.ff
         return n + 2 * self.vocab_size * d + d
 
     def kv_bytes_per_token(self, tp: int = 1, dtype_bytes: int = 2) -> int:
@@ -242,12 +272,18 @@ class LayeredConfig:
                 n += m.kv_heads * (2 * m.dim + m.vdim)
             elif m.kind == "latent_attention" and m.kv_from < 0:
                 n += m.kv_rank
+            elif m.kind == "rope_latent_attention" and m.kv_from < 0:
+                n += m.kv_rank + m.rot_dim
+            elif m.kind == "window_attention":
+                n += m.kv_heads * (m.dim + m.vdim)
         return max(1, n) * dtype_bytes
 
     def state_shapes(self, li: int) -> dict:
         """Per-sequence recurrent state of layer ``li`` besides cache pages and the input
         convolutions: name -> shape of one slot (fp32)."""
         m = self.layers[li].mixer
+        if self.token_shift:
+            return {"prev": (self.hidden,)}
         if m.kind == "wkv":
             return {"wkv": (m.heads, m.dim, m.dim), "prev": (self.hidden,)}
         if m.kind == "gla":
@@ -385,6 +421,103 @@ def bilolix_from_json(d: dict, name: str | None = None) -> LayeredConfig:
                          max_position=int(d.get("max_position", 8192)), loop=loop)
 
 
+def _rot_scaling(sc) -> tuple:
+    """``rot.scaling`` of a config.json -> MixerSpec.rot_scaling; the keys decide the rule."""
+    if not sc:
+        return ()
+    if "fast" in sc or "slow" in sc:
+        return ("yarn", float(sc["factor"]), float(sc["original"]), float(sc["fast"]), float(sc["slow"]))
+    return ("banded", float(sc["factor"]), float(sc["original"]), float(sc["low"]), float(sc["high"]))
+
+
+def nutitar_from_json(d: dict, name: str | None = None) -> LayeredConfig:
+    """config.json of a Nutitar checkpoint: vocab, width, norm.eps, embedding.scale,
+    residual_mult and ``layers``: type ``latent_attention`` (heads, dim, rot_dim, vdim, kv_rank,
+    scale, rot, optional kv_from), ``attention`` (heads, kv_heads, dim, vdim, scale, rot,
+    mask.size, mask.keep_first) or ``attention_2`` (heads, kv_heads, dim, scale, rot), each with
+    an ``mlp`` of kind ``dense`` (ff) or null."""
+    layers = []
+    for i, ly in enumerate(d["layers"]):
+        m, kind = ly["mixer"], ly["type"]
+        rot = m.get("rot") or {}
+        rd, rb = int(rot.get("dims", 0)), float(rot.get("base", 10000.0))
+        rs = _rot_scaling(rot.get("scaling"))
+        if kind == "latent_attention":
+            src = m.get("kv_from")
+            mixer = MixerSpec("rope_latent_attention", int(m["heads"]), 1, int(m["dim"]), int(m["vdim"]),
+                              float(m["scale"]), kv_rank=int(m["kv_rank"]),
+                              kv_from=-1 if src is None else int(src), rot_dims=rd, rot_base=rb,
+                              rot_dim=int(m["rot_dim"]), rot_scaling=rs)
+            if rd != mixer.rot_dim:
+                raise ValueError(f"layer {i}: the rotated part is rot_dim wide, rot.dims must equal it")
+            if mixer.kv_from >= 0:
+                if not 0 <= mixer.kv_from < i:
+                    raise ValueError(f"layer {i}: kv_from must name an earlier layer")
+                o = layers[mixer.kv_from].mixer
+                if o.kind != mixer.kind or o.kv_from >= 0 or o.kv_rank != mixer.kv_rank \
+                        or o.rot_dim != mixer.rot_dim:
+                    raise ValueError(f"layer {i}: layer {mixer.kv_from} holds no latent of rank "
+                                     f"{mixer.kv_rank} with a {mixer.rot_dim}-wide key part of its own")
+        elif kind in ("attention", "attention_2"):
+            second = kind == "attention_2"
+            mask = m.get("mask") or {}
+            mixer = MixerSpec("window_attention", int(m["heads"]), int(m["kv_heads"]), int(m["dim"]),
+                              int(m.get("vdim", m["dim"])), float(m["scale"]),
+                              window=int(mask.get("size", 0)), keep_first=int(mask.get("keep_first", 0)),
+                              rot_dims=rd, rot_base=rb, rot_scaling=rs,
+                              qk_norm="head" if second else "all",
+                              weights="softmax" if second else "sigmoid", bias=not second,
+                              v_is_k=second)
+            if mixer.heads % mixer.kv_heads:
+                raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+            if mixer.v_is_k and mixer.vdim != mixer.dim:
+                raise ValueError(f"layer {i}: values that are the keys have the keys' size")
+            if rd > mixer.dim:
+                raise ValueError(f"layer {i}: rot.dims must be at most dim")
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        if rd % 2:
+            raise ValueError(f"layer {i}: rot.dims must be even")
+        f = ly.get("mlp")
+        if f is not None and f.get("kind") != "dense":
+            raise ValueError(f"layer {i}: unknown feed-forward kind {f.get('kind')!r}")
+        layers.append(LayerSpec(mixer, None if f is None else MlpSpec("xielu", int(f["ff"]), 0.0)))
+    return LayeredConfig(name=name or d["architecture"].lower(), architecture=d["architecture"],
+                         vocab_size=int(d["vocab"]), hidden=int(d["width"]), layers=tuple(layers),
+                         rms_eps=float(d["norm"]["eps"]), embed_scale=float(d["embedding"]["scale"]),
+                         canon_taps=0, max_position=int(d.get("max_position", 8192)),
+                         residual_mult=float(d["residual_mult"]), token_shift=True)
+
+
+def nutitar_layers(order, heads, kv_heads, dim, vdim, ff, kv_rank=0, rot_dim=0, window=0,
+                   keep_first=0, rot_dims=None, rot_base=10000.0, yarn=(), banded=(), scale=None,
+                   latent_heads=None, latent_dim=None):
+    """Layers of the kinds named in ``order``: "l" latent attention with rotated key part, "s" one
+    that reads the nearest earlier latent layer's cache, "w" windowed sigmoid attention, "k"
+    softmax attention whose values are its keys."""
+    out, src = [], -1
+    rd = dim if rot_dims is None else rot_dims
+    lh, ld = latent_heads or heads, latent_dim or dim
+    for i, c in enumerate(order):
+        if c in "ls":
+            m = MixerSpec("rope_latent_attention", lh, 1, ld, vdim, scale or (ld + rot_dim) ** -0.5,
+                          kv_rank=kv_rank, kv_from=src if c == "s" else -1, rot_dims=rot_dim,
+                          rot_base=rot_base, rot_dim=rot_dim,
+                          rot_scaling=("yarn",) + tuple(yarn) if yarn else ())
+            src = i if c == "l" else src
+        elif c == "w":
+            m = MixerSpec("window_attention", heads, kv_heads, dim, vdim, scale or dim ** -0.5,
+                          window=window, keep_first=keep_first, rot_dims=rd, rot_base=rot_base,
+                          qk_norm="all", weights="sigmoid", bias=True)
+        else:
+            m = MixerSpec("window_attention", heads, kv_heads, dim, dim, scale or dim ** -0.5,
+                          rot_dims=rd, rot_base=rot_base,
+                          rot_scaling=("banded",) + tuple(banded) if banded else (),
+                          qk_norm="head", weights="softmax", v_is_k=True)
+        out.append(LayerSpec(m, MlpSpec("xielu", ff, 0.0) if ff else None))
+    return tuple(out)
+
+
 def bilolix_layers(order, heads, kv_heads, dim, vdim, ff, experts=0, top=0, expert_ff=0,
                    window=0, rot_dims=None, rot_base=10000.0, diff=0.5, tau=16.0, conv=4,
                    rec_heads=None, rec_kv_heads=None, rec_dim=None, moe_every=2):
@@ -448,11 +581,21 @@ TINY_BILOLIX = LayeredConfig("tiny-bilolix", architecture="Bilolix", vocab_size=
                                                    expert_ff=40, window=21, rot_dims=8,
                                                    rot_base=5000.0, diff=0.7, tau=8.0, conv=3,
                                                    rec_heads=4, rec_kv_heads=2))
-CONFIGS.update({c.name: c for c in (TINY_LIVISUN, LIVISUN_8B, TINY_NUMALORN, TINY_BILOLIX)})
+# every mixer kind once plus a layer that shares a latent cache; sizes that differ wherever the
+# design allows (dim != vdim, rot_dims < dim, kv_heads < heads, odd window, a layer without mlp)
+TINY_NUTITAR = LayeredConfig("tiny-nutitar", architecture="Nutitar", vocab_size=288, hidden=96,
+                             canon_taps=0, embed_scale=6.0, residual_mult=0.6, token_shift=True,
+                             layers=nutitar_layers("lwsk", 6, 2, 16, 24, 160, kv_rank=40, rot_dim=8,
+                                                   window=21, keep_first=3, rot_dims=12,
+                                                   rot_base=5000.0, yarn=(3.0, 64.0, 16.0, 2.0),
+                                                   banded=(3.0, 48.0, 1.0, 3.0), latent_heads=5,
+                                                   latent_dim=20))
+CONFIGS.update({c.name: c for c in (TINY_LIVISUN, LIVISUN_8B, TINY_NUMALORN, TINY_BILOLIX,
+                                    TINY_NUTITAR)})
 
 # config.json "architecture" -> reader
 ARCHITECTURES = {"Livisun": LayeredConfig.from_json, "Numalorn": numalorn_from_json,
-                 "Bilolix": bilolix_from_json}
+                 "Bilolix": bilolix_from_json, "Nutitar": nutitar_from_json}
 
 
 def load_config(path: str):

@@ -297,6 +297,8 @@ def load_layered_safetensors(path: str, cfg, device, dtype=torch.bfloat16) -> di
         return _numalorn_assemble(ck.full, lambda k: k in ck, cfg, device, dtype)
     if cfg.architecture == "Bilolix":
         return _bilolix_assemble(ck.full, lambda k: k in ck, cfg, device, dtype)
+    if cfg.architecture == "Nutitar":
+        return _nutitar_assemble(ck.full, lambda k: k in ck, cfg, device, dtype)
     w = {"embed": ck.full("embed").to(dtype).to(device), "lm_head": ck.full("head").to(dtype).to(device),
          "final_norm": ck.full("final.norm").float().to(device), "vocab_start": 0, "layers": []}
     for i, ly in enumerate(cfg.layers):
@@ -708,5 +710,155 @@ def init_bilolix_weights(cfg, device, dtype=torch.bfloat16, seed: int = 0,
 
 def bilolix_from_full(full: dict, cfg, device, dtype=torch.bfloat16) -> dict:
     w = _bilolix_assemble(lambda k: full[k], lambda k: k in full, cfg, device, dtype)
+    w["full"] = full
+    return w
+
+
+# --------------------------------------------------------------------------
+# Nutitar.  Checkpoint names:
+#   embed, head [V, d]; final.norm [d]; l<i>.norm1 [d] (stored around zero); l<i>.shift [d]
+#   latent attention: l<i>.mix.q [H*(dim+rot_dim), d]  .dkv [kv_rank+rot_dim, d]  .dkv.norm [kv_rank]
+#     (both absent with kv_from)  .uk [H*dim, kv_rank]  .uv [H*vdim, kv_rank]  .sink [H]  .g [H, d]
+#     .o [d, H*vdim]
+#   attention: l<i>.mix.q | k | v (+ .b)  .q.norm [H*dim]  .k.norm [G*dim]  .pb [H]  .o (+ .b)
+#   attention_2: l<i>.mix.q | k  .q.norm | .k.norm [dim]  .o
+#   feed-forward: l<i>.mlp.up [F, d]  .down [d, F]  .act [2]
+# Loaded layout per layer: one fused input projection "proj" (its bias "proj_b" in fp32), for
+# latent attention q | dkv | g rows with uk [H, dim, R] and uv^T [H, R, vdim] for the products
+# in the latent space; "mu" [2, d] = (0, shift): the token shift's mixes (the row itself in the
+# model's dtype, and the shifted row); "xi": the unit's two coefficients, formed once in float64.
+def _nutitar_assemble(get, has, cfg, device, dtype) -> dict:
+    import math
+
+    d = cfg.hidden
+
+    def mat(name, rows, cols):
+        t = get(name)
+        if tuple(t.shape) != (rows, cols):
+            raise ValueError(f"tensor {name}: shape {tuple(t.shape)}, expected {(rows, cols)}")
+        return t.to(dtype)
+
+    def vec(name, *shape):
+        t = get(name)
+        if tuple(t.shape) != tuple(shape):
+            raise ValueError(f"tensor {name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+        return t.float().contiguous().to(device)
+
+    def softplus(v):
+        return max(v, 0.0) + math.log1p(math.exp(-abs(v)))
+
+    V = cfg.vocab_size
+    w = {"embed": mat("embed", V, d).to(device), "lm_head": mat("head", V, d).to(device),
+         "final_norm": vec("final.norm", d), "vocab_start": 0, "layers": []}
+    for i, ly in enumerate(cfg.layers):
+        p, m, lw = f"l{i}.mix.", ly.mixer, LayerWeights()
+        lw["norm1"] = vec(f"l{i}.norm1", d)
+        shift = vec(f"l{i}.shift", d) if has(f"l{i}.shift") else torch.zeros(d, device=device)
+        lw["mu"] = torch.stack([torch.zeros_like(shift), shift]).contiguous()
+        H, G, dim, vd = m.heads, m.kv_heads, m.dim, m.vdim
+        if m.kind == "rope_latent_attention":
+            R, rd = m.kv_rank, m.rot_dim
+            parts = [mat(p + "q", H * (dim + rd), d)]
+            if m.kv_from < 0:
+                parts.append(mat(p + "dkv", R + rd, d))
+                lw["dkv_norm"] = vec(p + "dkv.norm", R)
+            parts.append(mat(p + "g", H, d))
+            lw["proj"] = torch.cat(parts, 0).contiguous().to(device)
+            lw["proj_b"] = None
+            lw["uk"] = mat(p + "uk", H * dim, R).view(H, dim, R).contiguous().to(device)
+            lw["uv_t"] = mat(p + "uv", H * vd, R).view(H, vd, R).transpose(1, 2).contiguous().to(device)
+            lw["sink"] = vec(p + "sink", H)
+            lw["o_b"] = None
+        elif m.kind == "window_attention":
+            names = ["q", "k"] + ([] if m.v_is_k else ["v"])
+            rows = {"q": H * dim, "k": G * dim, "v": G * vd}
+            lw["proj"] = torch.cat([mat(p + n, rows[n], d) for n in names], 0).contiguous().to(device)
+            lw["proj_b"] = torch.cat([vec(p + n + ".b", rows[n]) for n in names]).contiguous() \
+                if m.bias else None
+            if m.qk_norm == "all":
+                lw["qn"], lw["kn"] = vec(p + "q.norm", H * dim), vec(p + "k.norm", G * dim)
+            elif m.qk_norm == "head":
+                lw["qn"], lw["kn"] = vec(p + "q.norm", dim), vec(p + "k.norm", dim)
+            else:
+                lw["qn"] = lw["kn"] = None
+            lw["pb"] = vec(p + "pb", H) if m.weights == "sigmoid" else None
+            lw["o_b"] = vec(p + "o.b", d).to(dtype) if m.bias else None
+        else:
+            raise ValueError(f"layer {i}: no weights known for mixer {m.kind!r}")
+        lw["o"] = mat(p + "o", d, H * vd).contiguous().to(device)
+        f, q = ly.mlp, f"l{i}.mlp."
+        if f is not None:
+            lw["up"] = mat(q + "up", f.ff, d).contiguous().to(device)
+            lw["down"] = mat(q + "down", d, f.ff).contiguous().to(device)
+            a = vec(q + "act", 2).double().cpu()
+            lw["xi"] = (softplus(float(a[0])), 0.5 + softplus(float(a[1])))
+        w["layers"].append(lw)
+    return w
+
+
+def init_nutitar_weights(cfg, device, dtype=torch.bfloat16, seed: int = 0,
+                         keep_full: bool = True) -> dict:
+    """Seeded random Nutitar weights under the checkpoint's names (tests and benchmarks):
+    projections scaled so that activations stay O(1); shifts, sinks, biases, norm weights and
+    the unit's numbers away from their neutral values so that each shows in the logits.
+    ``keep_full`` False (benchmark sizes): drawn on the device, the name -> tensor dict is not
+    kept."""
+    d, full = cfg.hidden, {}
+
+    def rnd(name, shape, std, mean=0.0):
+        if keep_full:
+            t = _randn(shape, std, (seed, name), "cpu", torch.float32) + mean
+            full[name] = t.to(torch.bfloat16).float()
+        else:
+            full[name] = (_randn(shape, std, (seed, name), device, torch.float32) + mean).to(torch.bfloat16)
+        return full[name]
+
+    rnd("embed", (cfg.vocab_size, d), 1.0 / max(1.0, cfg.embed_scale))
+    rnd("head", (cfg.vocab_size, d), 2.0 * d ** -0.5)
+    rnd("final.norm", (d,), 0.2)
+    for i, ly in enumerate(cfg.layers):
+        p, m = f"l{i}.mix.", ly.mixer
+        H, G, dim, vd = m.heads, m.kv_heads, m.dim, m.vdim
+        rnd(f"l{i}.norm1", (d,), 0.2)
+        rnd(f"l{i}.shift", (d,), 0.25, 0.4)
+        if m.kind == "rope_latent_attention":
+            R, rd = m.kv_rank, m.rot_dim
+            rnd(p + "q", (H * (dim + rd), d), 2.0 * d ** -0.5)
+            if m.kv_from < 0:
+                rnd(p + "dkv", (R + rd, d), 2.0 * d ** -0.5)
+                rnd(p + "dkv.norm", (R,), 0.1, 1.0)
+            rnd(p + "uk", (H * dim, R), 2.0 * R ** -0.5)
+            rnd(p + "uv", (H * vd, R), R ** -0.5)
+            rnd(p + "sink", (H,), 1.0)
+            rnd(p + "g", (H, d), 2.0 * d ** -0.5)
+        else:
+            n = H * dim if m.qk_norm == "all" else dim
+            rnd(p + "q", (H * dim, d), 2.0 * d ** -0.5)
+            rnd(p + "k", (G * dim, d), 2.0 * d ** -0.5)
+            if m.qk_norm:
+                rnd(p + "q.norm", (n,), 0.2, 1.5)
+                rnd(p + "k.norm", (n if m.qk_norm == "head" else G * dim,), 0.2, 1.5)
+            if not m.v_is_k:
+                rnd(p + "v", (G * vd, d), d ** -0.5)
+            if m.bias:
+                rnd(p + "q.b", (H * dim,), 0.3)
+                rnd(p + "k.b", (G * dim,), 0.3)
+                rnd(p + "v.b", (G * vd,), 0.3)
+                rnd(p + "o.b", (d,), 0.3)
+            if m.weights == "sigmoid":
+                rnd(p + "pb", (H,), 1.0, -2.0)
+        rnd(p + "o", (d, H * vd), (H * vd) ** -0.5)
+        if ly.mlp is not None:
+            q = f"l{i}.mlp."
+            rnd(q + "up", (ly.mlp.ff, d), d ** -0.5)
+            rnd(q + "down", (d, ly.mlp.ff), ly.mlp.ff ** -0.5)
+            rnd(q + "act", (2,), 0.5, 0.3)
+    if not keep_full:
+        return _nutitar_assemble(lambda k: full.pop(k), lambda k: k in full, cfg, device, dtype)
+    return nutitar_from_full(full, cfg, device, dtype)
+
+
+def nutitar_from_full(full: dict, cfg, device, dtype=torch.bfloat16) -> dict:
+    w = _nutitar_assemble(lambda k: full[k], lambda k: k in full, cfg, device, dtype)
     w["full"] = full
     return w

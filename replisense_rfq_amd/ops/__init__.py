@@ -1182,13 +1182,13 @@ def attn_latent_mfma(q, pool, block_tables, q_start, q_len, kv_len, work_seq, wo
                               out, torch.zeros(q.shape[1]), sink, 0)
 
 
-def embed_rows(ids, table, out=None):
+def embed_rows(ids, table, out=None, scale: float = 1.0):
     out = torch.empty((ids.numel(), table.shape[1]), dtype=torch.float32, device=table.device) \
         if out is None else out
     if _gpu(table):
-        _native.mix_ops().embed_rows(ids, table, out)
+        _native.mix_ops().embed_rows(ids, table, out, float(scale))
     else:
-        ref.embed_rows(ids, table, out)
+        ref.embed_rows(ids, table, out, scale)
     return out
 
 
@@ -1287,13 +1287,15 @@ def softcap(x, cap: float):
 # recurrences, activated convolutions, softmax top-k routing (csrc/kernels/mix_diff_attn.hip,
 # mix_linrec.hip, mix_par.hip; same library).
 def residual_add_norm(x, y1=None, y2=None, shift=None, w=None, eps: float = 1e-5,
-                      offset: float = 0.0, out=None):
-    """x (fp32, in place) += y1 + y2 + shift (each optional, either dtype; shift is one fp32
-    row added to every row); with ``w``, ``out`` receives rms(x) * (w + offset)."""
+                      offset: float = 0.0, out=None, mult: float = 1.0):
+    """x (fp32, in place) += mult * (y1 + y2) + shift (each optional, either dtype; shift is one
+    fp32 row added to every row); with ``w``, ``out`` (either dtype) receives
+    rms(x) * (w + offset)."""
     if _gpu(x):
-        _native.mix_ops().residual_add_norm(x, y1, y2, shift, w, float(eps), float(offset), out)
+        _native.mix_ops().residual_add_norm(x, y1, y2, shift, w, float(eps), float(offset), out,
+                                            float(mult))
     else:
-        ref.residual_add_norm(x, y1, y2, shift, w, eps, offset, out)
+        ref.residual_add_norm(x, y1, y2, shift, w, eps, offset, out, mult)
     return out
 
 
@@ -1393,4 +1395,67 @@ def gelu_rows(x, out=None):
         _native.mix_ops().gelu_rows(x, out)
     else:
         ref.gelu_rows(x, out)
+    return out
+
+
+# ---------------------------------------------------------------------------
+# Scaled half-split rotation with projection norms, attention with a sliding window that keeps
+# the first tokens and softmax / sink / sigmoid weights, xIELU (csrc/kernels/mix_keep_attn.hip,
+# mix_keep_attn_mfma.hip, mix_par.hip; same library).
+def rotary_scaled_freq(rot_dims: int, base: float, scaling: tuple = (), device="cpu"):
+    return ref.rotary_scaled_freq(rot_dims, base, scaling, device)
+
+
+def qk_norm_rotary_append(proj, bias, q_norm_w, k_norm_w, norm_all: bool, k_norm_n: int, eps: float,
+                          positions, inv_freq, rot_mult: float, q_rot_off: int, k_rot_off: int,
+                          slot_mapping, k_cache, v_cache, H: int, G: int, qw: int, kw: int, vdim: int,
+                          v_mode: int, q_out):
+    if _gpu(proj):
+        _native.mix_ops().qk_norm_rotary_append(
+            proj, bias, q_norm_w, k_norm_w, bool(norm_all), int(k_norm_n), float(eps), positions,
+            inv_freq, float(rot_mult), int(q_rot_off), int(k_rot_off), slot_mapping, k_cache,
+            v_cache, H, G, qw, kw, vdim, int(v_mode), q_out)
+    else:
+        ref.qk_norm_rotary_append(proj, bias, q_norm_w, k_norm_w, norm_all, k_norm_n, eps, positions,
+                                  inv_freq, rot_mult, q_rot_off, k_rot_off, slot_mapping, k_cache,
+                                  v_cache, H, G, qw, kw, vdim, v_mode, q_out)
+    return q_out
+
+
+KEEP_QBLK = 32       # queries per work item of attn_keep_window (the scheduler's MIXQ_QBLK)
+KEEP_MFMA = os.environ.get("RFQ_KEEP_MFMA", "1") != "0"     # bf16: MFMA tiles where sizes fit
+
+
+def keep_mfma_ok(E: int, vdim: int, block: int = 32) -> bool:
+    """Whether the MFMA tiles of attn_keep_window cover these sizes (bf16 pages, GPU)."""
+    return bool(KEEP_MFMA and _native.mix_ops().keep_mfma_ok(E, vdim, block))
+
+
+def attn_keep_window(q, k_cache, v_cache, vdim: int, block_tables, q_start, q_len, kv_len, work_seq,
+                     work_qblk, head_bias, gate, out, scale: float, window: int = 0,
+                     keep_first: int = 0, sigmoid: bool = False, short_rows: int = 0,
+                     mfma: bool | None = None):
+    """Work items (sequence, block of KEEP_QBLK queries) as for attn_mixq_prefill.
+    ``short_rows`` > 0: every sequence has at most that many rows (a decode section); the
+    kernel then runs one workgroup per (sequence, key/value head) over one pass through the
+    pages where the sizes fit its LDS.  bf16 pages whose sizes the MFMA tiles cover run on them
+    unless ``mfma`` is False (the FMA kernels)."""
+    if _gpu(q):
+        _native.mix_ops().attn_keep_window(q, k_cache, v_cache, int(vdim), block_tables, q_start,
+                                           q_len, kv_len, work_seq, work_qblk, head_bias, gate, out,
+                                           float(scale), int(window), int(keep_first),
+                                           bool(sigmoid), int(short_rows),
+                                           KEEP_MFMA if mfma is None else bool(mfma))
+    else:
+        ref.attn_keep_window(q, k_cache, v_cache, vdim, block_tables, q_start, q_len, kv_len,
+                             head_bias, gate, out, scale, window, keep_first, sigmoid)
+    return out
+
+
+def xielu_rows(x, alpha_p: float, alpha_n: float, out=None):
+    out = torch.empty_like(x) if out is None else out
+    if _gpu(x):
+        _native.mix_ops().xielu_rows(x, float(alpha_p), float(alpha_n), out)
+    else:
+        ref.xielu_rows(x, alpha_p, alpha_n, out)
     return out

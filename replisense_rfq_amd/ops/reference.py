@@ -357,9 +357,9 @@ def glu_clamped(gate_up, limit: float, alpha: float, out) -> None:
 
 # --------------------------------------------------------------------------
 # Post-norm residual layers, latent attention, wkv recurrence, grouped sigmoid routing.
-def embed_rows(ids, table, out) -> None:
-    """out[t] = table[ids[t]] in fp32."""
-    out.copy_(table[ids.long()].float())
+def embed_rows(ids, table, out, scale: float = 1.0) -> None:
+    """out[t] = table[ids[t]] * scale in fp32."""
+    out.copy_(table[ids.long()].float() * scale)
 
 
 def post_norm_add(y, residual, w, mult: float, eps: float, out) -> None:
@@ -508,12 +508,15 @@ def moe_experts(h, ids, weights, w13, w2, base, out) -> None:
 # ---------------------------------------------------------------------------
 # Parallel-sublayer residual, rotary windowed differential attention, gated linear
 # recurrences (plain and delta rule), activated causal convolutions, softmax top-k routing.
-def residual_add_norm(x, y1, y2, shift, w, eps: float, offset: float, out) -> None:
-    """x (fp32, in place) += y1 + y2 + shift (each optional; shift is one row for all);
-    with ``w``: out = x / sqrt(mean(x^2) + eps) * (w + offset) in out's dtype."""
-    for y in (y1, y2, shift):
-        if y is not None:
-            x.add_(y.float())
+def residual_add_norm(x, y1, y2, shift, w, eps: float, offset: float, out,
+                      mult: float = 1.0) -> None:
+    """x (fp32, in place) += mult * (y1 + y2) + shift (each optional; shift is one row for
+    all); with ``w``: out = x / sqrt(mean(x^2) + eps) * (w + offset) in out's dtype."""
+    if y1 is not None or y2 is not None:
+        y = (y1.float() if y1 is not None else 0.0) + (y2.float() if y2 is not None else 0.0)
+        x.add_(y * mult if mult != 1.0 else y)
+    if shift is not None:
+        x.add_(shift.float())
     if w is not None:
         out.copy_((_rms(x, eps) * (w.float() + offset)).to(out.dtype))
 
@@ -700,3 +703,151 @@ def gelu_rows(x, out) -> None:
     """out = 0.5 x (1 + erf(x / sqrt 2)), computed in fp32."""
     xf = x.float()
     out.copy_((0.5 * xf * (1.0 + torch.erf(xf * 0.7071067811865476))).to(out.dtype))
+
+
+# ---------------------------------------------------------------------------
+# Scaled half-split rotation, projection norms, attention with a sliding window that keeps
+# the first tokens and softmax / sink / sigmoid weights, the xIELU unit.
+def rotary_scaled_freq(rot_dims: int, base: float, scaling: tuple = (), device="cpu"):
+    """(f [rot_dims / 2] fp32, multiplier of cos and sin).  f_i = base^(-2i / rot_dims), then by
+    ``scaling``:
+      ("yarn", factor, original, fast, slow): with dim(t) = rot_dims ln(original / (2 pi t)) /
+        (2 ln base), lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), rot_dims - 1) and
+        r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1): f_i (r_i / factor + 1 - r_i); the
+        multiplier is 0.1 ln(factor) + 1;
+      ("banded", factor, original, low, high): wavelengths 2 pi / f below original / high keep
+        f, above original / low get f / factor, between them the blend
+        (1 - s) f / factor + s f with s = (original f / (2 pi) - low) / (high - low).
+    Everything in float64, rounded once."""
+    n = rot_dims // 2
+    i = torch.arange(n, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / max(1, rot_dims))
+    mult = 1.0
+    if scaling and scaling[0] == "yarn":
+        _, factor, original, fast, slow = scaling
+
+        def dim_of(t):
+            return rot_dims * math.log(original / (2.0 * math.pi * t)) / (2.0 * math.log(base))
+
+        lo = max(math.floor(dim_of(fast)), 0)
+        hi = min(math.ceil(dim_of(slow)), rot_dims - 1)
+        r = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        f = f / factor * r + f * (1.0 - r)
+        mult = 0.1 * math.log(factor) + 1.0
+    elif scaling and scaling[0] == "banded":
+        _, factor, original, low, high = scaling
+        wl = 2.0 * math.pi / f
+        s = (original / wl - low) / (high - low)
+        mid = (1.0 - s) * f / factor + s * f
+        f = torch.where(wl < original / high, f, torch.where(wl > original / low, f / factor, mid))
+    elif scaling:
+        raise ValueError(f"unknown frequency scaling {scaling[0]!r}")
+    return f.float().to(device), float(mult)
+
+
+def _rotate_halves(x, positions, inv_freq, mult: float, off: int):
+    """Entries off + i and off + i + n (n = len(inv_freq)) of the last axis of x [T, ..., w]
+    turn by the angle position * f_i; cos and sin carry the factor ``mult`` (all fp32)."""
+    n = inv_freq.numel()
+    if n == 0:
+        return x
+    ang = positions.float()[:, None] * inv_freq.float()[None]
+    shape = (x.shape[0],) + (1,) * (x.dim() - 2) + (n,)
+    c, s = (torch.cos(ang) * mult).view(shape), (torch.sin(ang) * mult).view(shape)
+    y = x.clone()
+    u, v = x[..., off:off + n], x[..., off + n:off + 2 * n]
+    y[..., off:off + n] = u * c - v * s
+    y[..., off + n:off + 2 * n] = v * c + u * s
+    return y
+
+
+def qk_norm_rotary_append(proj, bias, q_norm_w, k_norm_w, norm_all: bool, k_norm_n: int, eps: float,
+                          positions, inv_freq, rot_mult: float, q_rot_off: int, k_rot_off: int,
+                          slot_mapping, k_cache, v_cache, H: int, G: int, qw: int, kw: int, vdim: int,
+                          v_mode: int, q_out) -> None:
+    """Rows of proj are q [H, qw] | k [G, kw] (| v [G, vdim] with v_mode 0); ``bias`` (fp32, the
+    row's width) is added first.  RMS norms with plain weights: over the whole q and the whole k
+    projection (``norm_all``; weights [H qw], [G kw]) or per head, q over its qw entries
+    (weight [qw]) and k over its leading ``k_norm_n`` entries (weight [k_norm_n]); a weight of
+    None means no norm.  Then the half-split rotation of entries rot_off .. rot_off + 2 n of
+    every head.  q goes to q_out [T, H, qw] fp32; k rows into k_cache [blocks, G, BS, kw];
+    values into v_cache [blocks, G, BS, vdim]: v_mode 0 the v columns, 1 the keys as projected
+    (before norm and rotation), 2 none."""
+    T = proj.shape[0]
+    if T == 0:
+        return
+    x = proj.float()
+    if bias is not None:
+        x = x + bias.float()
+    nq, nk = H * qw, G * kw
+    q, k = x[:, :nq], x[:, nq:nq + nk]
+    raw_k = k.reshape(T, G, kw)
+    if norm_all:
+        if q_norm_w is not None:
+            q = _rms(q, eps) * q_norm_w.float()
+        if k_norm_w is not None:
+            k = _rms(k, eps) * k_norm_w.float()
+        q, k = q.reshape(T, H, qw), k.reshape(T, G, kw)
+    else:
+        q, k = q.reshape(T, H, qw), k.reshape(T, G, kw).clone()
+        if q_norm_w is not None:
+            q = _rms(q, eps) * q_norm_w.float()
+        if k_norm_w is not None:
+            k[..., :k_norm_n] = _rms(k[..., :k_norm_n], eps) * k_norm_w.float()
+    q = _rotate_halves(q, positions[:T], inv_freq, rot_mult, q_rot_off)
+    k = _rotate_halves(k, positions[:T], inv_freq, rot_mult, k_rot_off)
+    q_out.copy_(q)
+    if k_cache is None or G == 0:
+        return
+    v = x[:, nq + nk:nq + nk + G * vdim].reshape(T, G, vdim) if v_mode == 0 else raw_k
+    BS = k_cache.shape[2]
+    for t in range(T):
+        s = int(slot_mapping[t])
+        if s >= 0:
+            k_cache[s // BS, :, s % BS] = k[t].to(k_cache.dtype)
+            if v_mode != 2:
+                v_cache[s // BS, :, s % BS] = v[t].to(v_cache.dtype)
+
+
+def attn_keep_window(q, k_cache, v_cache, vdim: int, block_tables, q_start, q_len, kv_len, head_bias,
+                     gate, out, scale: float, window: int, keep_first: int, sigmoid: bool) -> None:
+    """q [T, H, E] fp32; k_cache [blocks, G, BS, E]; the values are the first ``vdim`` entries
+    of v_cache's rows (which may be the key pages themselves).  Position i sees j <= i with
+    i - j < window or j < keep_first (window 0: every j <= i).  Weights: softmax over the
+    visible keys, with exp(head_bias[h]) added to the denominator when head_bias is given; or
+    (``sigmoid``) sigmoid(score + head_bias[h]) per visible key, not normalised.  ``gate``
+    [T, H]: the head's output is multiplied by sigmoid(gate).  out [T, H vdim]."""
+    H = q.shape[1]
+    G = k_cache.shape[1]
+    rep = H // G
+    for b in range(q_len.shape[0]):
+        ql, kl, t0 = int(q_len[b]), int(kv_len[b]), int(q_start[b])
+        if ql == 0:
+            continue
+        k = _gather_kv(k_cache, block_tables[b], kl).float().repeat_interleave(rep, 0)
+        v = _gather_kv(v_cache, block_tables[b], kl).float()[..., :vdim].repeat_interleave(rep, 0)
+        i = torch.arange(kl - ql, kl)[:, None]
+        j = torch.arange(kl)[None, :]
+        ok = j <= i
+        if window > 0:
+            ok = ok & ((i - j < window) | (j < keep_first))
+        s = torch.einsum("qhe,hke->hqk", q[t0:t0 + ql].float(), k) * scale
+        if sigmoid:
+            p = torch.sigmoid(s + head_bias.float()[:, None, None]) * ok[None]
+        else:
+            s = s.masked_fill(~ok[None], float("-inf"))
+            if head_bias is not None:
+                s = torch.cat([s, head_bias.float()[:, None, None].expand(H, ql, 1)], -1)
+            p = torch.softmax(s, -1)[..., :kl]
+        o = torch.einsum("hqk,hkd->qhd", p, v)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[t0:t0 + ql].float())[:, :, None]
+        out[t0:t0 + ql].copy_(o.reshape(ql, -1).to(out.dtype))
+
+
+def xielu_rows(x, alpha_p: float, alpha_n: float, out) -> None:
+    """z > 0: alpha_p z^2 + z / 2;  z <= 0: alpha_n (exp(z) - 1 - z) + z / 2, in fp32."""
+    z = x.float()
+    zn = torch.clamp(z, max=0.0)
+    out.copy_(torch.where(z > 0, alpha_p * z * z + 0.5 * z,
+                          alpha_n * (torch.expm1(zn) - zn) + 0.5 * zn).to(out.dtype))
