@@ -77,9 +77,9 @@ def parse():
     ap.add_argument("--arch-sizes", default="", help="--arch-compare: size classes, comma separated")
     ap.add_argument("--arch-models", default="",
                     help="--arch-compare: which of the two models to run (default both), comma separated; "
-                         "'kernels' (bilolix): only the per-kernel times")
+                         "'kernels' (bilolix, nutitar): only the per-kernel times")
     ap.add_argument("--arch-compare", default="",
-                    help="livisun | numalorn: instead of the RFQ workload, time prefill and decode "
+                    help="livisun | numalorn | bilolix | nutitar: instead of the RFQ workload, time prefill and decode "
                          "of the layer-list model beside the closest decoder at equal layer sizes "
                          "(replisense_rfq_amd/benchmarks/arch_compare.py); one JSON line")
     ap.add_argument("--time-budget", type=float, default=0.0,
@@ -367,8 +367,8 @@ def main():
     args = parse()
     t_start = time.perf_counter()
     if args.arch_compare:
-        if args.arch_compare not in ("livisun", "numalorn", "bilolix") or args.gpus != 1:
-            raise SystemExit("bench: --arch-compare livisun | numalorn | bilolix runs on one GPU")
+        if args.arch_compare not in ("livisun", "numalorn", "bilolix", "nutitar") or args.gpus != 1:
+            raise SystemExit("bench: --arch-compare livisun | numalorn | bilolix | nutitar runs on one GPU")
         from replisense_rfq_amd.benchmarks import arch_compare
 
         extra = {}
@@ -381,6 +381,10 @@ def main():
             from replisense_rfq_amd.benchmarks import arch_kernels
 
             extra["kernels"] = arch_kernels.run_bilolix(args)
+        if args.arch_compare == "nutitar" and (not args.arch_models or "kernels" in args.arch_models):
+            from replisense_rfq_amd.benchmarks import arch_kernels
+
+            extra["kernels"] = arch_kernels.run_nutitar(args)
         print(json.dumps({"metric": "arch_compare", "arch": args.arch_compare, "dtype": "bf16",
                           "data": "synthetic", **arch_compare.run(args), **extra}), flush=True)
         return

@@ -81,11 +81,11 @@ int launch_attn_keep_decode(bool, const float*, const void*, const void*, int64_
                             int, const int32_t*, const int32_t*, const int32_t*, int, int,
                             const float*, const void*, int64_t, void*, int64_t, float, int, int,
                             bool, int, int, int, int, int, hipStream_t);
-bool keep_mfma_ok(int, int, int);
-void launch_attn_keep_mfma(const float*, const void*, const void*, int64_t, const int32_t*, int,
+bool keep_mfma_ok(int, int, int, bool);
+bool launch_attn_keep_mfma(const float*, const void*, const void*, int64_t, const int32_t*, int,
                            const int32_t*, const int32_t*, const int32_t*, const int32_t*,
                            const int32_t*, int, const float*, const void*, int64_t, void*, int64_t,
-                           float, int, int, bool, int, int, int, int, int, hipStream_t);
+                           float, int, int, bool, int, int, int, int, int, bool, hipStream_t);
 void launch_xielu_rows(bool, const void*, int64_t, void*, int64_t, int, int, float, float,
                        hipStream_t);
 void launch_rotary_append(bool, const void*, int64_t, const int32_t*, const float*, int,
@@ -736,11 +736,15 @@ void attn_keep_window(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
               rows2d(out, T, (int64_t)H * vdim), "attn_keep_window: out [T, H vdim]");
   TORCH_CHECK(window >= 0 && keep_first >= 0, "attn_keep_window: window, keep_first");
   const float* hb = optf(head_bias, "head_bias", H);
-  const bool tiles = mfma && !f32 && rfqmix::keep_mfma_ok(E, (int)vdim, BS) && vrs % 8 == 0 &&
+  // the values are the leading entries of the key pages themselves
+  const bool shared = v_cache.data_ptr() == k_cache.data_ptr() && vrs == E;
+  const bool tiles = mfma && !f32 && rfqmix::keep_mfma_ok(E, (int)vdim, BS, shared) &&
+                     vrs % 8 == 0 && out.stride(0) % 4 == 0 &&
                      reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0 &&
                      reinterpret_cast<uintptr_t>(k_cache.data_ptr()) % 16 == 0 &&
-                     reinterpret_cast<uintptr_t>(v_cache.data_ptr()) % 16 == 0;
-  if (short_rows > 0 && !tiles) {
+                     reinterpret_cast<uintptr_t>(v_cache.data_ptr()) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(out.data_ptr()) % 8 == 0;
+  if (short_rows > 0) {
     // sequences of at most short_rows rows each (decode section): one workgroup per
     // (sequence, key/value head); falls through to the work items if the LDS is too small
     TORCH_CHECK(short_rows <= 65535 && G <= 65535, "attn_keep_window: short_rows");
@@ -757,7 +761,7 @@ void attn_keep_window(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
         (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
         i32p(kv_len, "kv_len", NB), i32p(work_seq, "work_seq", W), i32p(work_qblk, "work_qblk", W),
         W, hb, gp, gs, out.data_ptr(), out.stride(0), (float)scale, (int)window, (int)keep_first,
-        sigmoid, H, G, E, (int)vdim, BS, stream());
+        sigmoid, H, G, E, (int)vdim, BS, shared, stream());
     return;
   }
   const bool ok = rfqmix::launch_attn_keep_window(
@@ -769,8 +773,8 @@ void attn_keep_window(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
   TORCH_CHECK(ok, "attn_keep_window: value size too large for the LDS");
 }
 
-bool keep_mfma_ok(int64_t E, int64_t vdim, int64_t BS) {
-  return rfqmix::keep_mfma_ok((int)E, (int)vdim, (int)BS);
+bool keep_mfma_ok(int64_t E, int64_t vdim, int64_t BS, bool shared) {
+  return rfqmix::keep_mfma_ok((int)E, (int)vdim, (int)BS, shared);
 }
 
 void xielu_rows(const Tensor& x, double ap, double an, const Tensor& out) {

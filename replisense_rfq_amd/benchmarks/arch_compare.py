@@ -1,9 +1,10 @@
 """Prefill and decode throughput of a layer-list model beside the closest decoder of the
 framework at equal layer sizes: ``bench.py --arch-compare livisun`` (beside Llama),
 ``--arch-compare numalorn`` (beside the Mixtral-style sparse decoder: same width, head count,
-experts, choices per token and expert width) and ``--arch-compare bilolix`` (beside Numalorn:
+experts, choices per token and expert width), ``--arch-compare bilolix`` (beside Numalorn:
 same width, head count, experts and expert width; attention and recurrent layers alternate
-in both).
+in both) and ``--arch-compare nutitar`` (beside Bilolix with attention in every layer: same
+width, head counts and dense feed-forward width).
 
 Both run through the same engine (scheduler, paged cache, hipGraph decode steps), with
 random weights, a few layers of a real model's shape and a small vocabulary, so the numbers
@@ -79,6 +80,28 @@ def _bilolix_configs(name, d, H, G, E, top, F):
     return num, bil
 
 
+def _nutitar_configs(name, d, H, G, F):
+    """Bilolix and Nutitar at equal sizes, dense feed-forwards of width F in every layer.
+    Bilolix: differential attention in all four layers (two 64-wide maps per head, 128-wide
+    values, window 1,024).  Nutitar: a latent-attention layer (128 plain + 64 rotated query
+    dimensions per head over a 512-wide latent), a windowed sigmoid layer (128-wide heads,
+    window 1,024, 64 kept tokens), a layer that reads the first layer's latents, and a softmax
+    layer whose 128-wide keys are its values."""
+    from ..models.config import bilolix_layers, nutitar_layers
+
+    bil = LayeredConfig(f"cmp-bilolix-{name}", architecture="Bilolix", vocab_size=VOCAB, hidden=d,
+                        canon_taps=0, loop=(0, 0, 1),
+                        layers=bilolix_layers("aaaa"[:LAYERS], H, G, 64, 128, F, window=1024,
+                                              rot_dims=64, rot_base=5e5))
+    nut = LayeredConfig(f"cmp-nutitar-{name}", architecture="Nutitar", vocab_size=VOCAB, hidden=d,
+                        canon_taps=0, embed_scale=1.0, residual_mult=0.5, token_shift=True,
+                        layers=nutitar_layers("lwsk"[:LAYERS], H, G, 128, 128, F, kv_rank=512,
+                                              rot_dim=64, window=1024, keep_first=64, rot_dims=64,
+                                              rot_base=5e5, yarn=(4.0, 4096.0, 32.0, 1.0),
+                                              banded=(8.0, 8192.0, 1.0, 4.0)))
+    return bil, nut
+
+
 def _engine(mcfg, args, batch):
     from ..models import layered_model_class
     from ..models.llama import DecoderLM
@@ -93,6 +116,11 @@ def _engine(mcfg, args, batch):
         from ..models.weights import init_bilolix_weights
 
         w = init_bilolix_weights(mcfg, dev, torch.bfloat16, args.seed, keep_full=False)
+        model = layered_model_class(mcfg.architecture)(mcfg, dev, weights=w)
+    elif isinstance(mcfg, LayeredConfig) and mcfg.architecture == "Nutitar":
+        from ..models.weights import init_nutitar_weights
+
+        w = init_nutitar_weights(mcfg, dev, torch.bfloat16, args.seed, keep_full=False)
         model = layered_model_class(mcfg.architecture)(mcfg, dev, weights=w)
     elif isinstance(mcfg, LayeredConfig):
         model = layered_model_class(mcfg.architecture)(mcfg, dev, seed=args.seed)
@@ -134,9 +162,10 @@ def run(args) -> dict:
            "decode": [64, 128], "sizes": {}}
     only = [x for x in getattr(args, "arch_sizes", "").split(",") if x]
     arch = getattr(args, "arch_compare", "livisun")
-    base = {"livisun": "llama", "numalorn": "sparse", "bilolix": "numalorn"}[arch]
-    make = {"livisun": _configs, "numalorn": _moe_configs, "bilolix": _bilolix_configs}[arch]
-    for size in (SIZES if arch == "livisun" else MOE_SIZES):
+    base = {"livisun": "llama", "numalorn": "sparse", "bilolix": "numalorn", "nutitar": "bilolix"}[arch]
+    make = {"livisun": _configs, "numalorn": _moe_configs, "bilolix": _bilolix_configs,
+            "nutitar": _nutitar_configs}[arch]
+    for size in (SIZES if arch in ("livisun", "nutitar") else MOE_SIZES):
         name = size[0]
         if only and name not in only:
             continue

@@ -291,3 +291,126 @@ def run_bilolix(args) -> dict:
     _attention(32, 512, [600] * 64, [1] * 64, like_dec, "decode", mfma=True)
     res["decode_step_64_rows"] = {"bilolix": dec, "numalorn": like_dec}
     return res
+
+
+# ---------------------------------------------------------------------------
+# Nutitar's kernels (``bench.py --arch-compare nutitar``) beside Bilolix's like kernels in the
+# same run: 4096-wide layers, 32 heads over 8 key/value heads of 128, a 512-wide latent with a
+# 64-wide rotated key part, window 1,024 with 64 kept tokens.
+def _pages(lens, q_lens, G, kw, vw, g):
+    BS = 32
+    nblk = sum((n + BS - 1) // BS for n in lens) + 1
+    kc = (torch.randn(nblk, G, BS, kw, generator=g, device=DEV) * 0.5).bfloat16()
+    vc = None if vw == 0 else (torch.randn(nblk, G, BS, vw, generator=g, device=DEV) * 0.5).bfloat16()
+    maxb = (max(lens) + BS - 1) // BS
+    tables, at, slots = [], 0, []
+    for n, q in zip(lens, q_lens):
+        nb = (n + BS - 1) // BS
+        tables.append(list(range(at, at + nb)) + [nblk - 1] * (maxb - nb))
+        slots += [(at + p // BS) * BS + p % BS for p in range(n - q, n)]
+        at += nb
+    pos = torch.cat([torch.arange(n - q, n) for n, q in zip(lens, q_lens)]).to(torch.int32).to(DEV)
+    starts = [sum(q_lens[:i]) for i in range(len(lens))]
+    work = [(s, b) for s, n in enumerate(q_lens) for b in range((n + 31) // 32)]
+    meta = (_i32(tables), _i32(starts), _i32(q_lens), _i32(lens), _i32([w[0] for w in work]),
+            _i32([w[1] for w in work]))
+    return kc, vc, pos, _i32(slots), meta
+
+
+def _n_attention(kind, H, G, lens, q_lens, out, name, window=0, keep=0):
+    """kind: "window" (sigmoid, biased, norm over the projection), "keyval" (softmax, head
+    norms, values = keys) or "latent" (512 + 64 wide shared pages, sink, gate)."""
+    g = torch.Generator(device=DEV).manual_seed(3)
+    T = sum(q_lens)
+    short = ops.TALK_DECODE_MAX_ROWS if name == "decode" else 0
+    dim = 128
+    if kind == "latent":
+        R, rd = 512, 64
+        E, vd, Gk = R + rd, R, 1
+        kc, _, pos, sl, meta = _pages(lens, q_lens, 1, E, 0, g)
+        vc = kc
+        N = H * (dim + rd) + E + H
+        pr = (torch.randn(T, N, generator=g, device=DEV) * 0.5).bfloat16()
+        nw = torch.randn(R, generator=g, device=DEV)
+        inv, mult = ops.rotary_scaled_freq(rd, 5e5, ("yarn", 4.0, 4096.0, 32.0, 1.0), DEV)
+        qf = torch.empty(T, H, dim + rd, device=DEV)
+        t = _time(lambda: ops.qk_norm_rotary_append(pr, None, None, nw, False, R, 1e-5, pos, inv, mult, dim,
+                                                    R, sl, kc, None, H, 1, dim + rd, E, 0, 2, qf))
+        out[f"qk_norm_rotary_append latent ({name})"] = _entry(
+            t, T * (H * (dim + rd) + E) * 2 + T * H * (dim + rd) * 4 + T * E * 2, 0)
+        q = torch.randn(T, H, E, generator=g, device=DEV) * 0.3
+        bias = torch.randn(H, generator=g, device=DEV)
+        gate = pr[:, N - H:]
+        sig = False
+    else:
+        E, vd, Gk = dim, dim, G
+        kc, vc, pos, sl, meta = _pages(lens, q_lens, G, dim, dim, g)
+        second = kind == "keyval"
+        N = (H + G) * dim + (0 if second else G * dim)
+        pr = (torch.randn(T, N, generator=g, device=DEV) * 0.5).bfloat16()
+        pb = None if second else torch.randn(N, generator=g, device=DEV)
+        n = dim if second else H * dim
+        qn = torch.randn(n, generator=g, device=DEV)
+        kn = torch.randn(dim if second else G * dim, generator=g, device=DEV)
+        inv, mult = ops.rotary_scaled_freq(64, 5e5, (), DEV)
+        q = torch.empty(T, H, dim, device=DEV)
+        t = _time(lambda: ops.qk_norm_rotary_append(pr, pb, qn, kn, not second, dim, 1e-5, pos, inv, mult, 0,
+                                                    0, sl, kc, vc, H, G, dim, dim, dim, 1 if second else 0, q))
+        out[f"qk_norm_rotary_append {kind} ({name})"] = _entry(
+            t, T * N * 2 + T * H * dim * 4 + T * G * 2 * dim * 2, 0)
+        bias = None if second else torch.randn(H, generator=g, device=DEV) - 3.0
+        gate, sig = None, not second
+    o = torch.empty(T, H * vd, dtype=torch.bfloat16, device=DEV)
+    pairs = seen = 0
+    for n_, q_ in zip(lens, q_lens):
+        for p in range(n_ - q_, n_):
+            pairs += p + 1 if window == 0 else min(p + 1, window + min(keep, max(0, p + 1 - window)))
+        seen += n_ if window == 0 else min(n_, window + q_ - 1 + keep)
+    flops = (2.0 * E + 2.0 * vd) * H * pairs
+    nbytes = seen * Gk * (E + (0 if kind == "latent" else vd)) * 2 + T * H * (E * 4 + vd * 2)
+    bt, qs, ql, kl, ws, wq = meta
+    t = _time(lambda: ops.attn_keep_window(q, kc, vc, vd, bt, qs, ql, kl, ws, wq, bias, gate, o, E ** -0.5,
+                                           window, keep, sig, short_rows=short), reps=5, warm=2)
+    out[f"attn_keep_window {kind} ({name})"] = _entry(t, nbytes, flops)
+
+
+def _n_rows(T, d, lens, slots, out, first=0):
+    g = torch.Generator(device=DEV).manual_seed(0)
+    x = torch.randn(T, d, generator=g, device=DEV)
+    y1 = torch.randn(T, d, generator=g, device=DEV).bfloat16()
+    y2 = torch.randn(T, d, generator=g, device=DEV).bfloat16()
+    w = torch.randn(d, generator=g, device=DEV) * 0.3
+    hf = torch.empty(T, d, device=DEV)
+    out["residual_add_norm"] = _entry(
+        _time(lambda: ops.residual_add_norm(x, y1, y2, None, w, 1e-5, 1.0, hf, mult=0.5)), T * d * 16, 0)
+    mu = torch.rand(2, d, generator=g, device=DEV)
+    prev = torch.zeros(2 * 64, d, device=DEV)
+    rows = _runs(lens, slots, first)
+    mixes = torch.empty(2, T, d, dtype=torch.bfloat16, device=DEV)
+    out["token_shift_mix"] = _entry(_time(lambda: ops.token_shift_mix(hf, mu, prev, *rows, mixes)),
+                                    T * d * 8 + len(lens) * d * 8, 0)
+    F = 14336
+    u = torch.randn(T, F, generator=g, device=DEV).bfloat16()
+    o = torch.empty_like(u)
+    out["xielu_rows"] = _entry(_time(lambda: ops.xielu_rows(u, 0.8, 1.2, o)), T * F * 4, 0)
+
+
+def run_nutitar(args) -> dict:
+    torch.manual_seed(0)
+    d, H, G, window, keep = 4096, 32, 8, 1024, 64
+    res = {"width": d, "heads": [H, G], "head": 128, "latent": [512, 64], "window": [window, keep]}
+    for name, lens, q_lens, key in (("prefill", [2048, 600], [2048, 600], "prefill_step_rows"),
+                                    ("decode", [600] * 64, [1] * 64, "decode_step_64_rows")):
+        mine, like = {}, {}
+        T = sum(q_lens)
+        rl = [2048, 2048] if name == "prefill" else [1] * 64
+        sl = [0, 63] if name == "prefill" else list(range(64))
+        _n_rows(sum(rl), d, rl, sl, mine, 0 if name == "prefill" else 600)
+        _n_attention("window", H, G, lens, q_lens, mine, name, window, keep)
+        _n_attention("keyval", H, G, lens, q_lens, mine, name)
+        _n_attention("latent", H, G, lens, q_lens, mine, name)
+        _b_rows(sum(rl), d, like)
+        _b_attention(H, G, 64, 128, window, lens, q_lens, like, name)
+        _attention(32, 512, lens, q_lens, like, name, mfma=True)
+        res[key] = {"nutitar": mine, "bilolix": like, "rows": T}
+    return res

@@ -1426,9 +1426,10 @@ KEEP_QBLK = 32       # queries per work item of attn_keep_window (the scheduler'
 KEEP_MFMA = os.environ.get("RFQ_KEEP_MFMA", "1") != "0"     # bf16: MFMA tiles where sizes fit
 
 
-def keep_mfma_ok(E: int, vdim: int, block: int = 32) -> bool:
-    """Whether the MFMA tiles of attn_keep_window cover these sizes (bf16 pages, GPU)."""
-    return bool(KEEP_MFMA and _native.mix_ops().keep_mfma_ok(E, vdim, block))
+def keep_mfma_ok(E: int, vdim: int, block: int = 32, shared: bool = False) -> bool:
+    """Whether the MFMA tiles of attn_keep_window cover these sizes (bf16 pages, GPU);
+    ``shared``: the values are the leading entries of the key pages."""
+    return bool(KEEP_MFMA and _native.mix_ops().keep_mfma_ok(E, vdim, block, shared))
 
 
 def attn_keep_window(q, k_cache, v_cache, vdim: int, block_tables, q_start, q_len, kv_len, work_seq,
@@ -1438,8 +1439,8 @@ def attn_keep_window(q, k_cache, v_cache, vdim: int, block_tables, q_start, q_le
     """Work items (sequence, block of KEEP_QBLK queries) as for attn_mixq_prefill.
     ``short_rows`` > 0: every sequence has at most that many rows (a decode section); the
     kernel then runs one workgroup per (sequence, key/value head) over one pass through the
-    pages where the sizes fit its LDS.  bf16 pages whose sizes the MFMA tiles cover run on them
-    unless ``mfma`` is False (the FMA kernels)."""
+    pages where the sizes fit its LDS.  Otherwise bf16 pages whose sizes the MFMA tiles cover
+    run on them unless ``mfma`` is False (the FMA work-item kernel)."""
     if _gpu(q):
         _native.mix_ops().attn_keep_window(q, k_cache, v_cache, int(vdim), block_tables, q_start,
                                            q_len, kv_len, work_seq, work_qblk, head_bias, gate, out,
