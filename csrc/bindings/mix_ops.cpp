@@ -85,7 +85,8 @@ bool keep_mfma_ok(int, int, int, bool);
 bool launch_attn_keep_mfma(const float*, const void*, const void*, int64_t, const int32_t*, int,
                            const int32_t*, const int32_t*, const int32_t*, const int32_t*,
                            const int32_t*, int, const float*, const void*, int64_t, void*, int64_t,
-                           float, int, int, bool, int, int, int, int, int, bool, hipStream_t);
+                           float, int, int, bool, int, int, int, int, int, bool, int, int,
+                           hipStream_t);
 void launch_xielu_rows(bool, const void*, int64_t, void*, int64_t, int, int, float, float,
                        hipStream_t);
 void launch_rotary_append(bool, const void*, int64_t, const int32_t*, const float*, int,
@@ -744,10 +745,11 @@ void attn_keep_window(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
                      reinterpret_cast<uintptr_t>(k_cache.data_ptr()) % 16 == 0 &&
                      reinterpret_cast<uintptr_t>(v_cache.data_ptr()) % 16 == 0 &&
                      reinterpret_cast<uintptr_t>(out.data_ptr()) % 8 == 0;
-  if (short_rows > 0) {
+  TORCH_CHECK(short_rows >= 0 && short_rows <= 65535 && G <= 65535, "attn_keep_window: short_rows");
+  if (short_rows > 0 && !(tiles && H / G >= 16)) {
     // sequences of at most short_rows rows each (decode section): one workgroup per
-    // (sequence, key/value head); falls through to the work items if the LDS is too small
-    TORCH_CHECK(short_rows <= 65535 && G <= 65535, "attn_keep_window: short_rows");
+    // (sequence, key/value head) on the FMA kernel; groups of 16 heads or more fill the MFMA
+    // tiles' columns and run there; falls through if the LDS is too small
     const int kt = rfqmix::launch_attn_keep_decode(
         f32, f32p(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), vrs, i32p(bt, "block_tables", 0),
         (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
@@ -761,7 +763,7 @@ void attn_keep_window(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
         (int)bt.size(1), i32p(q_start, "q_start", NB), i32p(q_len, "q_len", NB),
         i32p(kv_len, "kv_len", NB), i32p(work_seq, "work_seq", W), i32p(work_qblk, "work_qblk", W),
         W, hb, gp, gs, out.data_ptr(), out.stride(0), (float)scale, (int)window, (int)keep_first,
-        sigmoid, H, G, E, (int)vdim, BS, shared, stream());
+        sigmoid, H, G, E, (int)vdim, BS, shared, NB, (int)short_rows, stream());
     return;
   }
   const bool ok = rfqmix::launch_attn_keep_window(

@@ -30,8 +30,62 @@ constexpr float kNegInfK = -__builtin_huge_valf();
 }  // namespace
 
 // ------------------------------------------------------------------ norm, rotation, append
+namespace {
+// CW consecutive values as floats: CW = 8 moves 16 bytes of bf16 (32 of fp32) per access
+template <int CW>
+__device__ __forceinline__ void ld_chunk(const float* p, float* f) {
+  if constexpr (CW == 8) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+  } else {
+    f[0] = *p;
+  }
+}
+template <int CW>
+__device__ __forceinline__ void ld_chunk(const bf16_t* p, float* f) {
+  if constexpr (CW == 8) {
+    const uint4 w = *reinterpret_cast<const uint4*>(p);
+    const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(u[i] << 16);
+      f[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+    }
+  } else {
+    f[0] = ldf(p);
+  }
+}
+template <int CW>
+__device__ __forceinline__ void st_chunk(float* p, const float* f) {
+  if constexpr (CW == 8) {
+    *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(f[4], f[5], f[6], f[7]);
+  } else {
+    *p = f[0];
+  }
+}
+template <int CW>
+__device__ __forceinline__ void st_chunk(bf16_t* p, const float* f) {
+  if constexpr (CW == 8) {
+    uint32_t u[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      bf16_t lo, hi;
+      stf(&lo, f[2 * i]);
+      stf(&hi, f[2 * i + 1]);
+      u[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+    }
+    *reinterpret_cast<uint4*>(p) = make_uint4(u[0], u[1], u[2], u[3]);
+  } else {
+    stf(p, f[0]);
+  }
+}
+}  // namespace
+
+// One workgroup per row; the row passes through LDS as floats.  CW = 8: every width, stride and
+// pointer is a multiple of 8 values / 16 bytes, a thread moves chunks of 8 neighbouring values.
 // LDS (floats): row[W] | fac[H + G] | cs[2 nrot] | scratch[16]
-template <typename T>
+template <typename T, int CW>
 __global__ __launch_bounds__(256) void qk_norm_rotary_append_kernel(
     const T* __restrict__ proj, int64_t stride, const float* __restrict__ bias,
     const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, int norm_all,
@@ -39,18 +93,28 @@ __global__ __launch_bounds__(256) void qk_norm_rotary_append_kernel(
     int nrot, float rot_mult, int q_rot_off, int k_rot_off, const int32_t* __restrict__ slots,
     T* __restrict__ k_cache, T* __restrict__ v_cache, int H, int G, int qw, int kw, int vdim,
     int v_mode, int BS, int64_t pool_slots, float* __restrict__ q_out) {
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   const int t = blockIdx.x, tid = threadIdx.x, nthr = blockDim.x;
   const int lane = tid & 63, wid = tid >> 6, nw = nthr >> 6;
   const int nq = H * qw, nk = G * kw;
   const int W = nq + nk + (v_mode == 0 ? G * vdim : 0);
   float* row = lds;
-  float* fac = row + W;
+  float* fac = row + ((W + 3) & ~3);
   float* cs = fac + H + G;
   float* scratch = cs + 2 * nrot;
 
   const T* src = proj + (int64_t)t * stride;
-  for (int c = tid; c < W; c += nthr) row[c] = ldf(src + c) + (bias != nullptr ? bias[c] : 0.f);
+  for (int c = tid * CW; c < W; c += nthr * CW) {
+    float f[CW];
+    ld_chunk<CW>(src + c, f);
+    if (bias != nullptr) {
+      float b[CW];
+      ld_chunk<CW>(bias + c, b);
+#pragma unroll
+      for (int i = 0; i < CW; ++i) f[i] += b[i];
+    }
+    st_chunk<CW>(row + c, f);
+  }
   const float p = (float)pos[t];
   for (int i = tid; i < nrot; i += nthr) {
     float sn, c;
@@ -65,9 +129,9 @@ __global__ __launch_bounds__(256) void qk_norm_rotary_append_kernel(
   // the values first: they are the keys as projected (mode 1) or the v columns (mode 0)
   if (keep && v_mode != 2) {
     const float* vs = v_mode == 0 ? row + nq + nk : row + nq;
-    for (int x = tid; x < G * vdim; x += nthr) {
+    for (int x = tid * CW; x < G * vdim; x += nthr * CW) {
       const int g = x / vdim, e = x - g * vdim;
-      stf(v_cache + (page_row + (int64_t)g * BS) * vdim + e, vs[x]);
+      st_chunk<CW>(v_cache + (page_row + (int64_t)g * BS) * vdim + e, vs + x);
     }
   }
   // norm factors
@@ -96,36 +160,41 @@ __global__ __launch_bounds__(256) void qk_norm_rotary_append_kernel(
   }
   __syncthreads();
   // norm in place (the values above were taken before it)
-  for (int c = tid; c < nq + nk; c += nthr) {
+  for (int c = tid * CW; c < nq + nk; c += nthr * CW) {
     const bool isq = c < nq;
-    const int y = isq ? c : c - nq;
-    const int width = isq ? qw : kw;
-    const int hd = y / width, e = y - hd * width;
     const float* wv = isq ? q_norm_w : k_norm_w;
     if (wv == nullptr) continue;
-    if (norm_all) {
-      row[c] *= fac[isq ? 0 : 1] * wv[y];
-    } else if (isq || e < k_norm_n) {
-      row[c] *= fac[isq ? hd : H + hd] * wv[e];
-    }
+    const int y = isq ? c : c - nq;
+    const int width = isq ? qw : kw;
+    const int hd = y / width, e = y - hd * width;
+    const float fc = norm_all ? fac[isq ? 0 : 1] : fac[isq ? hd : H + hd];
+    const float* wp = norm_all ? wv + y : wv + e;
+#pragma unroll
+    for (int i = 0; i < CW; ++i)
+      if (norm_all || isq || e + i < k_norm_n) row[c + i] *= fc * wp[i];
   }
   __syncthreads();
-  for (int c = tid; c < nq + nk; c += nthr) {
+  for (int c = tid * CW; c < nq + nk; c += nthr * CW) {
     const bool isq = c < nq;
     const int y = isq ? c : c - nq;
     const int width = isq ? qw : kw;
     const int hd = y / width, e = y - hd * width;
-    const int r = e - (isq ? q_rot_off : k_rot_off);
-    float v = row[c];
-    if (r >= 0 && r < 2 * nrot) {
-      const int i = r < nrot ? r : r - nrot;
-      const float cc = cs[2 * i], sn = cs[2 * i + 1];
-      v = r < nrot ? v * cc - row[c + nrot] * sn : v * cc + row[c - nrot] * sn;
+    const int r0 = e - (isq ? q_rot_off : k_rot_off);
+    float v[CW];
+#pragma unroll
+    for (int i = 0; i < CW; ++i) {
+      const int r = r0 + i;
+      v[i] = row[c + i];
+      if (r >= 0 && r < 2 * nrot) {
+        const int ii = r < nrot ? r : r - nrot;
+        const float cc = cs[2 * ii], sn = cs[2 * ii + 1];
+        v[i] = r < nrot ? v[i] * cc - row[c + i + nrot] * sn : v[i] * cc + row[c + i - nrot] * sn;
+      }
     }
     if (isq)
-      q_out[(int64_t)t * nq + c] = v;
+      st_chunk<CW>(q_out + (int64_t)t * nq + c, v);
     else if (keep)
-      stf(k_cache + (page_row + (int64_t)hd * BS) * kw + e, v);
+      st_chunk<CW>(k_cache + (page_row + (int64_t)hd * BS) * kw + e, v);
   }
 }
 
@@ -492,8 +561,8 @@ namespace {
 constexpr int kLdsMax = 160 * 1024;
 template <typename K>
 void allow_lds(K kernel) {
-  hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                      hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax);
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax);
 }
 }  // namespace
 
@@ -505,27 +574,34 @@ bool launch_qk_norm_rotary_append(bool f32, const void* proj, int64_t stride, co
                                   int T, int H, int G, int qw, int kw, int vdim, int v_mode, int BS,
                                   int64_t pool_slots, float* q_out, hipStream_t s) {
   const size_t W = (size_t)H * qw + (size_t)G * kw + (v_mode == 0 ? (size_t)G * vdim : 0);
-  const size_t lds = (W + H + G + 2 * (size_t)nrot + 16) * sizeof(float);
+  const size_t lds = (W + 4 + H + G + 2 * (size_t)nrot + 16) * sizeof(float);
   if (lds > (size_t)kLdsMax) return false;
   if (T == 0) return true;
   static bool attr = false;
   if (!attr) {
-    allow_lds(&qk_norm_rotary_append_kernel<float>);
-    allow_lds(&qk_norm_rotary_append_kernel<bf16_t>);
+    allow_lds(&qk_norm_rotary_append_kernel<float, 1>);
+    allow_lds(&qk_norm_rotary_append_kernel<bf16_t, 1>);
+    allow_lds(&qk_norm_rotary_append_kernel<float, 8>);
+    allow_lds(&qk_norm_rotary_append_kernel<bf16_t, 8>);
     attr = true;
   }
-  if (f32)
-    hipLaunchKernelGGL(qk_norm_rotary_append_kernel<float>, dim3(T), dim3(256), lds, s,
-                       (const float*)proj, stride, bias, q_norm_w, k_norm_w, (int)norm_all, k_norm_n,
-                       eps, pos, inv_freq, nrot, rot_mult, q_rot_off, k_rot_off, slots,
-                       (float*)k_cache, (float*)v_cache, H, G, qw, kw, vdim, v_mode, BS, pool_slots,
-                       q_out);
-  else
-    hipLaunchKernelGGL(qk_norm_rotary_append_kernel<bf16_t>, dim3(T), dim3(256), lds, s,
-                       (const bf16_t*)proj, stride, bias, q_norm_w, k_norm_w, (int)norm_all,
-                       k_norm_n, eps, pos, inv_freq, nrot, rot_mult, q_rot_off, k_rot_off, slots,
-                       (bf16_t*)k_cache, (bf16_t*)v_cache, H, G, qw, kw, vdim, v_mode, BS,
-                       pool_slots, q_out);
+  auto al16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool vec = qw % 8 == 0 && (G == 0 || kw % 8 == 0) && (v_mode == 2 || vdim % 8 == 0) &&
+                   stride % 8 == 0 && k_norm_n % 8 == 0 && al16(proj) && al16(bias) &&
+                   al16(k_cache) && al16(v_cache) && al16(q_out);
+#define QKN_GO(TT, CW)                                                                          \
+  hipLaunchKernelGGL((qk_norm_rotary_append_kernel<TT, CW>), dim3(T), dim3(256), lds, s,       \
+                     (const TT*)proj, stride, bias, q_norm_w, k_norm_w, (int)norm_all, k_norm_n, \
+                     eps, pos, inv_freq, nrot, rot_mult, q_rot_off, k_rot_off, slots,           \
+                     (TT*)k_cache, (TT*)v_cache, H, G, qw, kw, vdim, v_mode, BS, pool_slots, q_out)
+  if (f32) {
+    if (vec) QKN_GO(float, 8);
+    else QKN_GO(float, 1);
+  } else {
+    if (vec) QKN_GO(bf16_t, 8);
+    else QKN_GO(bf16_t, 1);
+  }
+#undef QKN_GO
   return true;
 }
 

@@ -12,6 +12,10 @@
 // registers while the current one is multiplied.  Pages between the kept first tokens and the
 // window are never read.
 //
+// Decode rows (DEC): a workgroup takes one row of a sequence at a time and its 16 columns per
+// wave are 16 HEADS of one key/value head, so the pages of a sequence are streamed once for 32
+// heads (latent attention: all heads share the one key head) instead of once per head pair.
+//
 //   S^T[key, query] = K[key, :] . Q[query, :]   v_mfma_f32_16x16x32_bf16, A = key rows from LDS,
 //                     B = the queries in registers as bf16 hi (+ lo for keys of up to 320
 //                     entries: they arrive in fp32 and are not rounded a second time)
@@ -44,8 +48,9 @@ __device__ __forceinline__ void split_bf16w(const float* f, s16x8& hi, s16x8& lo
 }  // namespace
 
 // DK = E / 32, DV = vdim / 16, HPW heads per workgroup, SHARED: values = leading entries of the
-// key rows, QLO: the queries' lo parts are multiplied too.
-template <int DK, int DV, int HPW, bool SHARED, bool QLO>
+// key rows, QLO: the queries' lo parts are multiplied too, DEC: decode rows (grid = sequences x
+// (key/value head, block of 32 heads) x rows in flight; no work lists).
+template <int DK, int DV, int HPW, bool SHARED, bool QLO, bool DEC>
 __global__ __launch_bounds__(128 * HPW) void attn_keep_mfma_kernel(
     const float* __restrict__ q, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, int64_t vrs, const int32_t* __restrict__ block_tables,
@@ -57,33 +62,38 @@ __global__ __launch_bounds__(128 * HPW) void attn_keep_mfma_kernel(
   constexpr int E = 32 * DK, vdim = 16 * DV, NT = 128 * HPW;
   constexpr int KRS = E + 8;                       // shorts per key row in LDS (+ 16 bytes)
   constexpr int VRS = SHARED ? KRS : vdim + 8;     // shorts per value row
-  const int s = work_seq[blockIdx.x];
+  const int s = DEC ? (int)blockIdx.x : work_seq[blockIdx.x];
   if (s < 0) return;
-  const int i0 = work_qblk[blockIdx.x] * WQB;
   const int ql = q_len[s];
-  if (i0 >= ql) return;
-  const int nq = min(WQB, ql - i0);
-  const int p0 = kv_len[s] - ql + i0;
-  const int plast = p0 + nq - 1;
-  const int jwin = window > 0 ? max(0, p0 - window + 1) : 0;
-  const int kf = window > 0 ? min(keep_first, jwin) : 0;     // kept keys before the window
   const int32_t* bt = block_tables + (int64_t)s * maxb;
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
-  const int sub = wid & 1;
-  const int hh = blockIdx.y * HPW + (wid >> 1);
-  const int g = (blockIdx.y * HPW) / (H / G);      // the workgroup's heads share one value head
   const int col = lane & 15, grp = lane >> 4;
-  const int row = sub * 16 + col;                  // this lane's query of the block
-  const int pi = p0 + row;
-  const bool qlive = row < nq;
-
+  const int rep = H / G;
+  // prompt rows: columns are 16 queries of head hh; decode rows: 16 heads of one row
+  const int per_g = (rep + 32 * HPW - 1) / (32 * HPW);
+  const int ho = DEC ? ((int)blockIdx.y % per_g) * 32 * HPW + wid * 16 + col : 0;
+  const int g = DEC ? (int)blockIdx.y / per_g : ((int)blockIdx.y * HPW) / rep;
+  const int hh = DEC ? g * rep + min(ho, rep - 1) : (int)blockIdx.y * HPW + (wid >> 1);
+  const int i0 = DEC ? 0 : work_qblk[blockIdx.x] * WQB;
+  if (!DEC && i0 >= ql) return;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   short* Ks = reinterpret_cast<short*>(smem);      // [32][KRS]
   short* Vs = SHARED ? Ks : Ks + WBS * KRS;        // [32][VRS]
 
+  for (int r = DEC ? (int)blockIdx.z : 0; r < (DEC ? ql : 1); r += DEC ? (int)gridDim.z : 1) {
+  const int nq = DEC ? 1 : min(WQB, ql - i0);
+  const int p0 = kv_len[s] - ql + (DEC ? r : i0);
+  const int plast = p0 + nq - 1;
+  const int jwin = window > 0 ? max(0, p0 - window + 1) : 0;
+  const int kf = window > 0 ? min(keep_first, jwin) : 0;     // kept keys before the window
+  const int row = DEC ? r : (wid & 1) * 16 + col;  // this lane's query of the run / block
+  const int pi = DEC ? p0 : p0 + row;
+  const bool qlive = DEC ? ho < rep : row < nq;
+  const int64_t t = q_start[s] + i0 + row;
+
   s16x8 qhi[DK], qlo[QLO ? DK : 1];
   {
-    const float* qp = q + ((int64_t)(q_start[s] + i0 + row) * H + hh) * E + grp * 8;
+    const float* qp = q + (t * H + hh) * E + grp * 8;
 #pragma unroll
     for (int ks = 0; ks < DK; ++ks) {
       float f[8];
@@ -243,19 +253,20 @@ __global__ __launch_bounds__(128 * HPW) void attn_keep_mfma_kernel(
     }
     pg = pg_next;
   }
-  if (!qlive) return;
-  // lane (col, grp) holds value channels 16 m + 4 grp .. + 3 of its query: 8-byte stores
-  const int64_t t = q_start[s] + i0 + row;
-  float mul = sigmoid ? 1.f : (lrun > 0.f ? 1.0f / lrun : 0.f);
-  if (gate != nullptr) mul /= 1.0f + __expf(-ldf(gate + t * gate_stride + hh));
-  bf16_t* orow = out + t * out_stride + (int64_t)hh * vdim + grp * 4;
+  // lane (col, grp) holds value channels 16 m + 4 grp .. + 3 of its column: 8-byte stores
+  if (qlive) {
+    float mul = sigmoid ? 1.f : (lrun > 0.f ? 1.0f / lrun : 0.f);
+    if (gate != nullptr) mul /= 1.0f + __expf(-ldf(gate + t * gate_stride + hh));
+    bf16_t* orow = out + t * out_stride + (int64_t)hh * vdim + grp * 4;
 #pragma unroll
-  for (int m = 0; m < DV; ++m) {
-    bf16_t b[4];
+    for (int m = 0; m < DV; ++m) {
+      bf16_t b[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) stf(&b[i], o[m][i] * mul);
-    *reinterpret_cast<uint2*>(orow + m * 16) =
-        make_uint2((uint32_t)b[0] | ((uint32_t)b[1] << 16), (uint32_t)b[2] | ((uint32_t)b[3] << 16));
+      for (int i = 0; i < 4; ++i) stf(&b[i], o[m][i] * mul);
+      *reinterpret_cast<uint2*>(orow + m * 16) =
+          make_uint2((uint32_t)b[0] | ((uint32_t)b[1] << 16), (uint32_t)b[2] | ((uint32_t)b[3] << 16));
+    }
+  }
   }
 }
 
@@ -290,21 +301,27 @@ struct KeepArgs {
   int window, keep_first;
   bool sigmoid;
   int H, G;
+  int NA, short_rows;      // decode rows: sequences, and the most rows any of them has (0: work items)
   hipStream_t s;
 };
 
-template <int DK, int DV, int HPW, bool SHARED>
+template <int DK, int DV, int HPW, bool SHARED, bool DEC>
 static void launch_keep_mfma_one(const KeepArgs& a) {
   constexpr bool QLO = DK <= 10;       // wider keys: the queries' registers go to the accumulators
   constexpr int E = 32 * DK, vdim = 16 * DV;
   const size_t lds = (size_t)(WBS * (E + 8) + (SHARED ? 0 : WBS * (vdim + 8))) * 2;
   static bool attr = false;
   if (!attr) {
-    hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_keep_mfma_kernel<DK, DV, HPW, SHARED, QLO>),
-                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    (void)hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&attn_keep_mfma_kernel<DK, DV, HPW, SHARED, QLO, DEC>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     attr = true;
   }
-  hipLaunchKernelGGL((attn_keep_mfma_kernel<DK, DV, HPW, SHARED, QLO>), dim3(a.W, a.H / HPW),
+  const int rep = a.H / a.G;
+  const dim3 grid = DEC ? dim3(a.NA, a.G * ((rep + 32 * HPW - 1) / (32 * HPW)),
+                               a.short_rows < 4 ? a.short_rows : 4)
+                        : dim3(a.W, a.H / HPW);
+  hipLaunchKernelGGL((attn_keep_mfma_kernel<DK, DV, HPW, SHARED, QLO, DEC>), grid,
                      dim3(128 * HPW), lds, a.s, a.q, (const bf16_t*)a.k_cache,
                      (const bf16_t*)a.v_cache, a.vrs, a.bt, a.maxb, a.q_start, a.q_len, a.kv_len,
                      a.work_seq, a.work_qblk, a.head_bias, (const bf16_t*)a.gate, a.gate_stride,
@@ -314,8 +331,9 @@ static void launch_keep_mfma_one(const KeepArgs& a) {
 
 template <int DK, int DV, bool SHARED>
 static void launch_keep_mfma_heads(const KeepArgs& a) {
-  if ((a.H / a.G) % 2 == 0) launch_keep_mfma_one<DK, DV, 2, SHARED>(a);
-  else launch_keep_mfma_one<DK, DV, 1, SHARED>(a);
+  if (a.short_rows > 0) launch_keep_mfma_one<DK, DV, 1, SHARED, true>(a);
+  else if ((a.H / a.G) % 2 == 0) launch_keep_mfma_one<DK, DV, 2, SHARED, false>(a);
+  else launch_keep_mfma_one<DK, DV, 1, SHARED, false>(a);
 }
 
 bool launch_attn_keep_mfma(const float* q, const void* k_cache, const void* v_cache, int64_t vrs,
@@ -324,12 +342,13 @@ bool launch_attn_keep_mfma(const float* q, const void* k_cache, const void* v_ca
                            const int32_t* work_qblk, int W, const float* head_bias,
                            const void* gate, int64_t gate_stride, void* out, int64_t out_stride,
                            float scale, int window, int keep_first, bool sigmoid, int H, int G,
-                           int E, int vdim, int BS, bool shared, hipStream_t s) {
+                           int E, int vdim, int BS, bool shared, int NA, int short_rows,
+                           hipStream_t s) {
   if (!keep_mfma_ok(E, vdim, BS, shared)) return false;
-  if (W == 0) return true;
+  if (short_rows > 0 ? NA == 0 : W == 0) return true;
   const KeepArgs a{q, k_cache, v_cache, vrs, bt, maxb, q_start, q_len, kv_len, work_seq, work_qblk,
                    W, head_bias, gate, gate_stride, out, out_stride, scale, window, keep_first,
-                   sigmoid, H, G, s};
+                   sigmoid, H, G, NA, short_rows, s};
   const int DK = E / 32, DV = vdim / 16;
   if (shared) {
     if (DK == 3) launch_keep_mfma_heads<3, 4, true>(a);

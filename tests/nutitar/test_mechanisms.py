@@ -463,7 +463,8 @@ def test_two_sequences_one_launch(device):
 @pytest.mark.parametrize("H,G,E,vdim,shared", [(4, 2, 32, 32, False), (2, 1, 64, 128, False),
                                                (8, 2, 128, 64, False), (3, 3, 64, 64, False),
                                                (4, 1, 96, 64, True), (8, 1, 160, 128, True),
-                                               (3, 1, 576, 512, True)])
+                                               (3, 1, 576, 512, True), (16, 1, 96, 64, True),
+                                               (40, 2, 64, 64, False), (48, 1, 160, 128, True)])
 @pytest.mark.parametrize("window,keep", [(0, 0), (1, 0), (31, 3), (32, 33), (33, 1), (100, 40)])
 @pytest.mark.parametrize("kind", ["softmax", "sink", "sigmoid"])
 def test_attention_on_mfma_tiles(H, G, E, vdim, shared, window, keep, kind):
@@ -483,6 +484,9 @@ def test_attention_on_mfma_tiles(H, G, E, vdim, shared, window, keep, kind):
     args = (q, k, None if shared else v, vdim, sections, scale, window, keep, bias, gate, kind == "sigmoid")
     got = _attend("cuda", *args, dtype=torch.bfloat16, mfma=True)
     fma = _attend("cuda", *args, dtype=torch.bfloat16, mfma=False)
+    # decoded rows of groups of 16 heads or more: the tiles' columns are heads
+    dec = _attend("cuda", *args, dtype=torch.bfloat16, mfma=True, short=True)
+    close(dec, want, 6e-3 * (2.0 if E > 320 else 1.0))
     close(got, want, 6e-3 * (2.0 if E > 320 else 1.0))       # bf16 output
     # keys wider than 320 entries meet queries rounded to bf16 (no lo part)
     loose = 4.0 if E > 320 else 1.0
@@ -507,3 +511,16 @@ def test_mfma_tiles_see_the_window_edge_and_the_kept_tokens(window, sigmoid):
         got = _attend("cuda", q, k, v, vdim, [(0, L)], 1.0, window, keep, bias, None, sigmoid,
                       dtype=torch.bfloat16, mfma=True)
         assert (float(got[L - 1, 0]) > 50.0) == seen, (window, j, float(got[L - 1, 0]))
+    # the same through the decode rows' form (16 heads of one key head are the columns)
+    H = 16
+    for j, seen in ((L - window, True), (L - window - 1, False), (keep - 1, True), (keep, False)):
+        q = torch.randn(L, H, dim, generator=g) * 0.1
+        k = (torch.randn(L, G, dim, generator=g) * 0.1).bfloat16().float()
+        v = torch.randn(L, G, vdim, generator=g).bfloat16().float()
+        q[L - 1, :, 0] = 3.0
+        k[j, 0, 0] = 3.0
+        v[j, 0] = 100.0
+        hb = torch.full((H,), -4.0) if sigmoid else None
+        got = _attend("cuda", q, k, v, vdim, [(0, L - 1), (L - 1, 1)], 1.0, window, keep, hb, None, sigmoid,
+                      dtype=torch.bfloat16, mfma=True, short=True)
+        assert (float(got[L - 1, 0]) > 50.0) == seen and (float(got[L - 1, 15 * vdim]) > 50.0) == seen

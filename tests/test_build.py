@@ -21,7 +21,11 @@ def test_layer_list_kernel_library_builds_and_loads():
     torch.ops.load_library(str(so))
     for op in ("embed_sinusoid", "sandwich_norm", "canon_conv", "head_norm_append",
                "attn_talk_decode", "attn_mixq_prefill", "attn_mix_mfma", "glu_clamped",
-               "mixq_mfma_ok"):
+               "mixq_mfma_ok", "qk_norm_rotary_append", "attn_keep_window", "xielu_rows",
+               "keep_mfma_ok"):
         assert hasattr(torch.ops.rfq_mix, op), op
+    assert torch.ops.rfq_mix.keep_mfma_ok(128, 128, 32, False)
+    assert torch.ops.rfq_mix.keep_mfma_ok(576, 512, 32, True)
+    assert not torch.ops.rfq_mix.keep_mfma_ok(48, 48, 32, False)
     assert torch.ops.rfq_mix.mixq_mfma_ok(32, 8, 128, 128, 32)
     assert not torch.ops.rfq_mix.mixq_mfma_ok(6, 3, 24, 40, 32)
