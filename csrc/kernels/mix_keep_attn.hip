@@ -103,7 +103,9 @@ __global__ __launch_bounds__(256) void qk_norm_rotary_append_kernel(
   float* cs = fac + H + G;
   float* scratch = cs + 2 * nrot;
 
+  // the row into LDS; with whole-projection norms the squares are summed on the way
   const T* src = proj + (int64_t)t * stride;
+  float sq = 0.f, sk = 0.f;
   for (int c = tid * CW; c < W; c += nthr * CW) {
     float f[CW];
     ld_chunk<CW>(src + c, f);
@@ -114,6 +116,13 @@ __global__ __launch_bounds__(256) void qk_norm_rotary_append_kernel(
       for (int i = 0; i < CW; ++i) f[i] += b[i];
     }
     st_chunk<CW>(row + c, f);
+    if (norm_all) {
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < CW; ++i) ss += f[i] * f[i];
+      if (c < nq) sq += ss;
+      else if (c < nq + nk) sk += ss;
+    }
   }
   const float p = (float)pos[t];
   for (int i = tid; i < nrot; i += nthr) {
@@ -122,30 +131,26 @@ __global__ __launch_bounds__(256) void qk_norm_rotary_append_kernel(
     cs[2 * i] = c * rot_mult;
     cs[2 * i + 1] = sn * rot_mult;
   }
-  __syncthreads();
-  const int32_t slot = slots[t];
-  const bool keep = G > 0 && slot >= 0 && slot < pool_slots;
-  const int64_t page_row = keep ? ((int64_t)(slot / BS) * G) * BS + slot % BS : 0;   // + g * BS
-  // the values first: they are the keys as projected (mode 1) or the v columns (mode 0)
-  if (keep && v_mode != 2) {
-    const float* vs = v_mode == 0 ? row + nq + nk : row + nq;
-    for (int x = tid * CW; x < G * vdim; x += nthr * CW) {
-      const int g = x / vdim, e = x - g * vdim;
-      st_chunk<CW>(v_cache + (page_row + (int64_t)g * BS) * vdim + e, vs + x);
-    }
-  }
-  // norm factors
+  // norm factors: fac[0], fac[1] (whole projections) or one per head
   if (norm_all) {
-    float sq = 0.f, sk = 0.f;
-    for (int c = tid; c < nq; c += nthr) sq += row[c] * row[c];
-    for (int c = tid; c < nk; c += nthr) sk += row[nq + c] * row[nq + c];
-    sq = block_sum(sq, scratch);
-    sk = block_sum(sk, scratch);
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    if (lane == 0) {
+      scratch[wid] = sq;
+      scratch[8 + wid] = sk;
+    }
+    __syncthreads();
     if (tid == 0) {
-      fac[0] = q_norm_w != nullptr ? 1.0f / sqrtf(sq / (float)nq + eps) : 1.f;
-      fac[1] = k_norm_w != nullptr && nk > 0 ? 1.0f / sqrtf(sk / (float)nk + eps) : 1.f;
+      float a = 0.f, b = 0.f;
+      for (int w = 0; w < nw; ++w) {
+        a += scratch[w];
+        b += scratch[8 + w];
+      }
+      fac[0] = q_norm_w != nullptr ? 1.0f / sqrtf(a / (float)nq + eps) : 1.f;
+      fac[1] = k_norm_w != nullptr && nk > 0 ? 1.0f / sqrtf(b / (float)nk + eps) : 1.f;
     }
   } else {
+    __syncthreads();
     for (int hd = wid; hd < H + G; hd += nw) {
       const bool isq = hd < H;
       const float* hv = isq ? row + hd * qw : row + nq + (hd - H) * kw;
@@ -159,36 +164,41 @@ __global__ __launch_bounds__(256) void qk_norm_rotary_append_kernel(
     }
   }
   __syncthreads();
-  // norm in place (the values above were taken before it)
-  for (int c = tid * CW; c < nq + nk; c += nthr * CW) {
-    const bool isq = c < nq;
-    const float* wv = isq ? q_norm_w : k_norm_w;
-    if (wv == nullptr) continue;
-    const int y = isq ? c : c - nq;
-    const int width = isq ? qw : kw;
-    const int hd = y / width, e = y - hd * width;
-    const float fc = norm_all ? fac[isq ? 0 : 1] : fac[isq ? hd : H + hd];
-    const float* wp = norm_all ? wv + y : wv + e;
-#pragma unroll
-    for (int i = 0; i < CW; ++i)
-      if (norm_all || isq || e + i < k_norm_n) row[c + i] *= fc * wp[i];
+  const int32_t slot = slots[t];
+  const bool keep = G > 0 && slot >= 0 && slot < pool_slots;
+  const int64_t page_row = keep ? ((int64_t)(slot / BS) * G) * BS + slot % BS : 0;   // + g * BS
+  // the values: the keys as projected (mode 1) or the v columns (mode 0), neither normed nor rotated
+  if (keep && v_mode != 2) {
+    const float* vs = v_mode == 0 ? row + nq + nk : row + nq;
+    for (int x = tid * CW; x < G * vdim; x += nthr * CW) {
+      const int g = x / vdim, e = x - g * vdim;
+      st_chunk<CW>(v_cache + (page_row + (int64_t)g * BS) * vdim + e, vs + x);
+    }
   }
-  __syncthreads();
+  // q and k: norm factor and weight, then the rotation (the partner entry is normed on the way)
   for (int c = tid * CW; c < nq + nk; c += nthr * CW) {
     const bool isq = c < nq;
     const int y = isq ? c : c - nq;
     const int width = isq ? qw : kw;
     const int hd = y / width, e = y - hd * width;
+    const float* wv = isq ? q_norm_w : k_norm_w;
+    const int nn = wv == nullptr ? 0 : (norm_all || isq ? width : k_norm_n);   // normed entries of a head
+    const float fc = norm_all ? fac[isq ? 0 : 1] : fac[isq ? hd : H + hd];
+    const float* wp = wv == nullptr ? nullptr : (norm_all ? wv + (y - e) : wv);  // the head's weights
     const int r0 = e - (isq ? q_rot_off : k_rot_off);
     float v[CW];
 #pragma unroll
     for (int i = 0; i < CW; ++i) {
-      const int r = r0 + i;
+      const int ei = e + i, r = r0 + i;
       v[i] = row[c + i];
+      if (ei < nn) v[i] *= fc * wp[ei];
       if (r >= 0 && r < 2 * nrot) {
         const int ii = r < nrot ? r : r - nrot;
+        const int ej = r < nrot ? ei + nrot : ei - nrot;
+        float u = row[c + i + (ej - ei)];
+        if (ej < nn) u *= fc * wp[ej];
         const float cc = cs[2 * ii], sn = cs[2 * ii + 1];
-        v[i] = r < nrot ? v[i] * cc - row[c + i + nrot] * sn : v[i] * cc + row[c + i - nrot] * sn;
+        v[i] = r < nrot ? v[i] * cc - u * sn : v[i] * cc + u * sn;
       }
     }
     if (isq)
