@@ -554,16 +554,19 @@ __global__ __launch_bounds__(256) void attn_keep_decode_kernel(
 }
 
 // ------------------------------------------------------------------ xIELU
-template <typename T>
+template <typename T, int CW>
 __global__ __launch_bounds__(256) void xielu_rows_kernel(const T* __restrict__ x, int64_t xs,
                                                          T* __restrict__ out, int64_t os, int F,
                                                          float ap, float an) {
   const int t = blockIdx.x;
-  const int c = blockIdx.y * 256 + threadIdx.x;
+  const int c = (blockIdx.y * 256 + threadIdx.x) * CW;
   if (c >= F) return;
-  const float z = ldf(x + (int64_t)t * xs + c);
-  const float y = z > 0.f ? ap * z * z + 0.5f * z : an * (expm1f(z) - z) + 0.5f * z;
-  stf(out + (int64_t)t * os + c, y);
+  float z[CW], y[CW];
+  ld_chunk<CW>(x + (int64_t)t * xs + c, z);
+#pragma unroll
+  for (int i = 0; i < CW; ++i)
+    y[i] = z[i] > 0.f ? ap * z[i] * z[i] + 0.5f * z[i] : an * (expm1f(z[i]) - z[i]) + 0.5f * z[i];
+  st_chunk<CW>(out + (int64_t)t * os + c, y);
 }
 
 // ------------------------------------------------------------------ launchers
@@ -693,13 +696,21 @@ int launch_attn_keep_decode(bool f32, const float* q, const void* k_cache, const
 void launch_xielu_rows(bool f32, const void* x, int64_t xs, void* out, int64_t os, int T, int F,
                        float ap, float an, hipStream_t s) {
   if (T == 0 || F == 0) return;
-  const dim3 grid(T, (F + 255) / 256);
-  if (f32)
-    hipLaunchKernelGGL(xielu_rows_kernel<float>, grid, dim3(256), 0, s, (const float*)x, xs,
-                       (float*)out, os, F, ap, an);
-  else
-    hipLaunchKernelGGL(xielu_rows_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)x, xs,
-                       (bf16_t*)out, os, F, ap, an);
+  const bool vec = F % 8 == 0 && xs % 8 == 0 && os % 8 == 0 &&
+                   reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const int per = vec ? 2048 : 256;
+  const dim3 grid(T, (F + per - 1) / per);
+#define XI_GO(TT, CW)                                                                        \
+  hipLaunchKernelGGL((xielu_rows_kernel<TT, CW>), grid, dim3(256), 0, s, (const TT*)x, xs,  \
+                     (TT*)out, os, F, ap, an)
+  if (f32) {
+    if (vec) XI_GO(float, 8);
+    else XI_GO(float, 1);
+  } else {
+    if (vec) XI_GO(bf16_t, 8);
+    else XI_GO(bf16_t, 1);
+  }
+#undef XI_GO
 }
 
 }  // namespace rfqmix

@@ -448,8 +448,8 @@ def nutitar_from_json(d: dict, name: str | None = None) -> LayeredConfig:
                               float(m["scale"]), kv_rank=int(m["kv_rank"]),
                               kv_from=-1 if src is None else int(src), rot_dims=rd, rot_base=rb,
                               rot_dim=int(m["rot_dim"]), rot_scaling=rs)
-            if rd != mixer.rot_dim:
-                raise ValueError(f"layer {i}: the rotated part is rot_dim wide, rot.dims must equal it")
+            if rd > mixer.rot_dim:
+                raise ValueError(f"layer {i}: rot.dims must be at most rot_dim, the rotated part's width")
             if mixer.kv_from >= 0:
                 if not 0 <= mixer.kv_from < i:
                     raise ValueError(f"layer {i}: kv_from must name an earlier layer")

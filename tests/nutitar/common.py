@@ -19,7 +19,7 @@ def yarn(factor=3.0, original=40, fast=8.0, slow=1.0):
     return {"factor": factor, "original": original, "fast": fast, "slow": slow}
 
 
-def banded(factor=4.0, original=64, low=1.0, high=4.0):
+def banded(factor=5.0, original=64, low=1.0, high=6.0):
     return {"factor": factor, "original": original, "low": low, "high": high}
 
 
