@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void qk_norm_rotary_append_kernel(
   const int W = nq + nk + (v_mode == 0 ? G * vdim : 0);
   float* row = lds;
   float* fac = row + ((W + 3) & ~3);
-  float* cs = fac + H + G;
+  float* cs = fac + ((H + G + 3) & ~3);
   float* scratch = cs + 2 * nrot;
 
   // the row into LDS; with whole-projection norms the squares are summed on the way
@@ -151,16 +151,19 @@ __global__ __launch_bounds__(256) void qk_norm_rotary_append_kernel(
     }
   } else {
     __syncthreads();
-    for (int hd = wid; hd < H + G; hd += nw) {
+    // sixteen lanes per head: sixteen heads of the row are summed at a time
+    const int sub = tid & 15, ngrp = nthr >> 4;
+    for (int hd = tid >> 4; hd < H + G; hd += ngrp) {
       const bool isq = hd < H;
       const float* hv = isq ? row + hd * qw : row + nq + (hd - H) * kw;
       const int n = isq ? qw : k_norm_n;
       const bool normed = isq ? q_norm_w != nullptr : k_norm_w != nullptr;
       float ss = 0.f;
       if (normed)
-        for (int e = lane; e < n; e += 64) ss += hv[e] * hv[e];
-      ss = wave_sum(ss);
-      if (lane == 0) fac[hd] = normed ? 1.0f / sqrtf(ss / (float)n + eps) : 1.f;
+        for (int e = sub; e < n; e += 16) ss += hv[e] * hv[e];
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      if (sub == 0) fac[hd] = normed ? 1.0f / sqrtf(ss / (float)n + eps) : 1.f;
     }
   }
   __syncthreads();
@@ -175,7 +178,9 @@ __global__ __launch_bounds__(256) void qk_norm_rotary_append_kernel(
       st_chunk<CW>(v_cache + (page_row + (int64_t)g * BS) * vdim + e, vs + x);
     }
   }
-  // q and k: norm factor and weight, then the rotation (the partner entry is normed on the way)
+  // q and k: norm factor and weight, then the rotation (the partner entry is normed on the way).
+  // CW = 8: the normed width, the rotation's offset and its half are multiples of 8, so a chunk
+  // lies wholly inside or outside each of them and its partner chunk is one 32-byte LDS read.
   for (int c = tid * CW; c < nq + nk; c += nthr * CW) {
     const bool isq = c < nq;
     const int y = isq ? c : c - nq;
@@ -187,18 +192,48 @@ __global__ __launch_bounds__(256) void qk_norm_rotary_append_kernel(
     const float* wp = wv == nullptr ? nullptr : (norm_all ? wv + (y - e) : wv);  // the head's weights
     const int r0 = e - (isq ? q_rot_off : k_rot_off);
     float v[CW];
+    if constexpr (CW == 8) {
+      ld_chunk<8>(row + c, v);
+      if (e < nn) {
+        float w8[8];
+        ld_chunk<8>(wp + e, w8);
 #pragma unroll
-    for (int i = 0; i < CW; ++i) {
-      const int ei = e + i, r = r0 + i;
-      v[i] = row[c + i];
-      if (ei < nn) v[i] *= fc * wp[ei];
-      if (r >= 0 && r < 2 * nrot) {
-        const int ii = r < nrot ? r : r - nrot;
-        const int ej = r < nrot ? ei + nrot : ei - nrot;
-        float u = row[c + i + (ej - ei)];
-        if (ej < nn) u *= fc * wp[ej];
-        const float cc = cs[2 * ii], sn = cs[2 * ii + 1];
-        v[i] = r < nrot ? v[i] * cc - u * sn : v[i] * cc + u * sn;
+        for (int i = 0; i < 8; ++i) v[i] *= fc * w8[i];
+      }
+      if (r0 >= 0 && r0 < 2 * nrot) {
+        const bool first = r0 < nrot;
+        const int off = first ? nrot : -nrot, ii = first ? r0 : r0 - nrot;
+        float u[8], c8[8], s8[8];
+        ld_chunk<8>(row + c + off, u);
+        if (e + off < nn) {
+          float w8[8];
+          ld_chunk<8>(wp + e + off, w8);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) u[i] *= fc * w8[i];
+        }
+        ld_chunk<8>(cs + 2 * ii, c8);                 // (cos, sin) pairs ii .. ii + 3
+        ld_chunk<8>(cs + 2 * ii + 8, s8);             // pairs ii + 4 .. ii + 7
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float cc = i < 4 ? c8[2 * i] : s8[2 * (i - 4)];
+          const float sn = i < 4 ? c8[2 * i + 1] : s8[2 * (i - 4) + 1];
+          v[i] = first ? v[i] * cc - u[i] * sn : v[i] * cc + u[i] * sn;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < CW; ++i) {
+        const int ei = e + i, r = r0 + i;
+        v[i] = row[c + i];
+        if (ei < nn) v[i] *= fc * wp[ei];
+        if (r >= 0 && r < 2 * nrot) {
+          const int ii = r < nrot ? r : r - nrot;
+          const int ej = r < nrot ? ei + nrot : ei - nrot;
+          float u = row[c + i + (ej - ei)];
+          if (ej < nn) u *= fc * wp[ej];
+          const float cc = cs[2 * ii], sn = cs[2 * ii + 1];
+          v[i] = r < nrot ? v[i] * cc - u * sn : v[i] * cc + u * sn;
+        }
       }
     }
     if (isq)
@@ -587,7 +622,7 @@ bool launch_qk_norm_rotary_append(bool f32, const void* proj, int64_t stride, co
                                   int T, int H, int G, int qw, int kw, int vdim, int v_mode, int BS,
                                   int64_t pool_slots, float* q_out, hipStream_t s) {
   const size_t W = (size_t)H * qw + (size_t)G * kw + (v_mode == 0 ? (size_t)G * vdim : 0);
-  const size_t lds = (W + 4 + H + G + 2 * (size_t)nrot + 16) * sizeof(float);
+  const size_t lds = (W + 4 + H + G + 4 + 2 * (size_t)nrot + 16) * sizeof(float);
   if (lds > (size_t)kLdsMax) return false;
   if (T == 0) return true;
   static bool attr = false;
@@ -600,8 +635,9 @@ bool launch_qk_norm_rotary_append(bool f32, const void* proj, int64_t stride, co
   }
   auto al16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
   const bool vec = qw % 8 == 0 && (G == 0 || kw % 8 == 0) && (v_mode == 2 || vdim % 8 == 0) &&
-                   stride % 8 == 0 && k_norm_n % 8 == 0 && al16(proj) && al16(bias) &&
-                   al16(k_cache) && al16(v_cache) && al16(q_out);
+                   stride % 8 == 0 && k_norm_n % 8 == 0 && nrot % 8 == 0 && q_rot_off % 8 == 0 &&
+                   k_rot_off % 8 == 0 && al16(proj) && al16(bias) && al16(q_norm_w) &&
+                   al16(k_norm_w) && al16(k_cache) && al16(v_cache) && al16(q_out);
 #define QKN_GO(TT, CW)                                                                          \
   hipLaunchKernelGGL((qk_norm_rotary_append_kernel<TT, CW>), dim3(T), dim3(256), lds, s,       \
                      (const TT*)proj, stride, bias, q_norm_w, k_norm_w, (int)norm_all, k_norm_n, \

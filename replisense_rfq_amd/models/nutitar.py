@@ -142,10 +142,11 @@ class NutitarLM:
                                   self.cfg.rms_eps, m.positions[:T], lw["inv_freq"], lw["rot_mult"],
                                   dim, R, m.slot_mapping[:T], pool if own else None, None, H,
                                   1 if own else 0, dim + rd, R + rd, 0, 2, qf)
-        # the plain query part carried into the latent space, fp32 (a score operand), beside
-        # the rotated part: one (R + rd)-wide query per head
-        qn = qf[:, :, :dim].transpose(0, 1)
-        qa = ops.bmm_f32(qn if dt == torch.float32 else qn.to(dt), lw["uk"])        # [H, T, R]
+        # the plain query part (untouched by the kernel above: read as the projection left it)
+        # carried into the latent space, fp32 (a score operand), beside the rotated part: one
+        # (R + rd)-wide query per head
+        qn = pr[:, :nq].unflatten(1, (H, dim + rd))[:, :, :dim].transpose(0, 1)
+        qa = ops.bmm_f32(qn, lw["uk"])                                              # [H, T, R]
         qfull = torch.cat([qa.transpose(0, 1), qf[:, :, dim:]], -1)
         lat = torch.empty((T, H * R), dtype=dt, device=dev)
         self._attend(m, qfull, pool, pool, R, lw["sink"], gate, lat, mx)
