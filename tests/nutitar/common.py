@@ -75,11 +75,12 @@ ODD = config([latent(3, 6, 6, 10, 14, dense(18), scaling=yarn(2.0, 30, 6.0, 2.0)
               keyval(2, 1, 14, 10, None, scaling=banded(2.0, 30, 1.0, 3.0)),
               latent(2, 10, 6, 6, 14, dense(22), kv_from=0, scaling=yarn(2.0, 30, 6.0, 2.0))],
              vocab=53, width=36)
-# sizes the MFMA tiles cover (bf16 on the GPU)
+# sizes the MFMA tiles cover (bf16 on the GPU); sixteen heads over one key head: decoded rows
+# take the heads-as-columns form
 WIDE = config([window(8, 2, 32, 32, 40, 5, 16, dense(64), scale=0.2),
                keyval(4, 4, 64, 64, dense(64), scale=0.15, scaling=banded()),
                latent(4, 32, 32, 32, 64, dense(64), scale=0.15, scaling=yarn()),
-               latent(8, 32, 32, 16, 64, None, scale=0.15, scaling=yarn(), kv_from=2)],
+               latent(16, 32, 32, 16, 64, None, scale=0.15, scaling=yarn(), kv_from=2)],
               width=64, vocab=90)
 
 
